@@ -2,5 +2,6 @@ from .spec import PartSpec, SubLayerSpec, LayerSpec, ScheduleEntry, ModelSpec, C
 from .llama import LlamaConfig
 from .manirax import ManiraxConfig
 from .risonex import RisonexConfig
+from .dupolorn import DupolornConfig
 
-__all__ = ["PartSpec", "SubLayerSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig", "ManiraxConfig", "RisonexConfig"]
+__all__ = ["PartSpec", "SubLayerSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig", "ManiraxConfig", "RisonexConfig", "DupolornConfig"]

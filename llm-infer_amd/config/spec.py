@@ -61,10 +61,13 @@ class ScheduleEntry:
     """One run of a layer.  ``cache_from`` names an earlier entry of the schedule whose
     cache this run reads instead of keeping one of its own.  ``before``: a part of the "stream" registry that
     is run on the residual stream first (``forward(x, x0, ctx) -> x`` with x0 the embedding's output); entries
-    whose ``before`` specs are equal share one part, and so its tensors."""
+    whose ``before`` specs are equal share one part, and so its tensors.  ``after``: a part of the same registry
+    that makes the stream's next value from all its values so far (``forward_after(history, n, out, ctx)``, history
+    [runs, T, width] holding the embedding's output and the result of every run that such a part followed)."""
     layer: int
     cache_from: int | None = None
     before: PartSpec | None = None     # a "stream" part that rewrites the residual stream before this run
+    after: PartSpec | None = None      # a "stream" part that forms the stream's next value from all values so far
 
 
 @dataclass(frozen=True)

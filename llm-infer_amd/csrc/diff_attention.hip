@@ -10,7 +10,8 @@
 // accumulator elements of two lanes), then O_m^T += V^T P_m^T with the accumulators' own order of the keys, in which the
 // page holds the values.  A weight enters the second product as the sum of two 16-bit numbers (its rounding and the
 // rounding of the remainder), so that the product sees 16 bits of it.  At the end o = O_1 / l_1 - lambda O_2 / l_2,
-// divided by its root mean square over the value size and multiplied by out_scale.
+// divided by its root mean square over the value size and multiplied by out_scale.  `sink` not null: every map's sum
+// of weights also counts exp(sink[head]), a score with no key and no value that is not scaled.
 #include "common.h"
 
 #ifndef MAP_DIM
@@ -31,7 +32,8 @@ template <class T, int MAPS, bool PROMPT>
 __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, const int* __restrict__ tile_t0, const int* __restrict__ tile_n, int H, int G,
-    int dv, float scale, int block, int window, float lambda, float out_eps, float out_scale, int split) {
+    int dv, float scale, int block, int window, float lambda, float out_eps, float out_scale, int split,
+    const float* __restrict__ sink) {
     typedef typename Vec<T>::v8 v8;
     constexpr int D16 = MAP_DIM / 16, KW = MAPS * MAP_DIM, DVB = VALUE_DIM / 32;
     extern __shared__ float lds[];
@@ -222,6 +224,19 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
             }
         }
     }
+    if (sink) {
+        // the sink joins every map's sum as one more weight, exp(sink - maximum), with nothing to add to the output
+        const float s2 = sink[h] * 1.4426950408889634f;
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a) {
+            const float M = fmaxf(m[a], s2), f = __builtin_amdgcn_exp2f(m[a] - M);
+            l[a] = l[a] * f + __builtin_amdgcn_exp2f(s2 - M);
+#pragma unroll
+            for (int b = 0; b < DVB; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[a][b][r] *= f;
+        }
+    }
     // o = O_1 / l_1 - lambda O_2 / l_2 for this lane's query; its values lie in this lane and in lane ^ 32
     float ss = 0.f;
 #pragma unroll
@@ -259,7 +274,7 @@ extern "C" int li_diffattn_value_dim() { return VALUE_DIM; }
 extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages, const void* v_pages, int64_t page_stride,
                            const int* page_table, int max_pages, const int* pos, const int* tok_slot, const int* tile_t0,
                            const int* tile_n, int n_tiles, int H, int G, int maps, int dv, float scale, int block, int window,
-                           float lambda, float out_eps, float out_scale, hipStream_t stream) {
+                           float lambda, float out_eps, float out_scale, const float* sink, hipStream_t stream) {
     if (n_tiles <= 0) return LI_OK;
     if (H <= 0 || G <= 0 || H % G || dv <= 0 || dv > VALUE_DIM || block < 0 || window < 0) return LI_BAD_ARG;
     if (maps < 1 || maps > 2 || (dt != DT_F16 && dt != DT_BF16)) return LI_UNSUPPORTED;
@@ -273,7 +288,7 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
     const int threads = split ? 256 : 64 * heads;
     const size_t lds = split ? (size_t)4 * maps * (2 + VALUE_DIM) * sizeof(float) : 0;
 #define GO1(T, M, P) diff_attn_mfma_kernel<T, M, P><<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, \
-                                                                          tile_n, H, G, dv, scale, block, window, lambda, out_eps, out_scale, split)
+                                                                          tile_n, H, G, dv, scale, block, window, lambda, out_eps, out_scale, split, sink)
 #define GO(T, M) do { if (split) GO1(T, M, false); else GO1(T, M, true); } while (0)
     if (dt == DT_F16) { if (maps == 1) GO(f16, 1); else GO(f16, 2); }
     else { if (maps == 1) GO(bf16, 1); else GO(bf16, 2); }

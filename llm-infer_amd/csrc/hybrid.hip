@@ -73,19 +73,20 @@ extern "C" int li_concat_cast(const float* a, const float* b, void* out, int dt,
 }
 
 // ---------------------------------------------------------------------------
-// out = act(in), float32 in, type T out.  act: 0 gelu (erf), 1 gelu (tanh), 2 silu.
+// out = act(in), float32 in, type T out.  act: 0 gelu (erf), 1 gelu (tanh), 2 silu, 3 the square of relu.
 // ---------------------------------------------------------------------------
 template <class T>
 __global__ void activation_kernel(const float* __restrict__ in, T* __restrict__ out, int64_t n, int act) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const float z = in[i];
-    out[i] = from_f32<T>(act == 0 ? gelu_erff_(z) : (act == 1 ? gate_activation(z, true) : siluf_(z)));
+    const float r = fmaxf(z, 0.f);
+    out[i] = from_f32<T>(act == 0 ? gelu_erff_(z) : (act == 1 ? gate_activation(z, true) : (act == 2 ? siluf_(z) : r * r)));
 }
 
 extern "C" int li_activation(const float* in, void* out, int dt, int64_t n, int act, hipStream_t stream) {
     if (n <= 0) return LI_OK;
-    if (act < 0 || act > 2) return LI_BAD_ARG;
+    if (act < 0 || act > 3) return LI_BAD_ARG;
     DISPATCH_T(dt, (activation_kernel<T><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(in, (T*)out, n, act)));
     LI_CHECK_LAUNCH();
     return LI_OK;
@@ -163,18 +164,19 @@ extern "C" int li_qk_norm_store(const float* qkv, int stride, int col0, const fl
 // A token at position p sees the keys lo .. p with lo = p - p % block (block 0: lo = 0; window w > 0: lo is at
 // least p - w + 1).  Each of `maps` (1 or 2) maps is a softmax of its own over scores q_m . k_m * scale; with a_m
 // the maps' weighted sums of the SAME values,  o = a_1 - lambda a_2  (one map: o = a_1).  out_eps >= 0: o is
-// divided by its root mean square over dv and multiplied by out_scale.  Scores, weights, sums: float32.
+// divided by its root mean square over dv and multiplied by out_scale.  `sink` not null: every map's sum of weights
+// also counts exp(sink[head]), a score with no key and no value that is not scaled.  Scores, weights, sums: float32.
 // The waves of the workgroup take the tiles of 64 keys in turn, a lane a key; each keeps a running maximum and
 // sum per map (online softmax) and its share of the output, and the shares are merged through LDS in wave order.
 // ---------------------------------------------------------------------------
 #define DA_WAVES 4
-#define DA_MAXV 4          // dv <= 64 * DA_MAXV
+#define DA_MAXV 8          // dv <= 64 * DA_MAXV
 
 template <class T, int MAPS>
 __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, int H, int G, int d, int dv, float scale, int block, int window, float lambda,
-    float out_eps, float out_scale) {
+    float out_eps, float out_scale, const float* __restrict__ sink) {
     extern __shared__ float lds[];
     const int DP = round_up(d, 16), KW = MAPS * DP;
     float* sq = lds;                                   // [KW]
@@ -262,7 +264,8 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
                 for (int a = 0; a < MAPS; ++a) {
                     float M = sm[a];
                     for (int w = 1; w < DA_WAVES; ++w) M = fmaxf(M, sm[w * MAPS + a]);
-                    float L = 0.f, O = 0.f;
+                    if (sink) M = fmaxf(M, sink[h]);
+                    float L = sink ? expf(sink[h] - M) : 0.f, O = 0.f;
                     for (int w = 0; w < DA_WAVES; ++w) {
                         const float mw = sm[w * MAPS + a];
                         const float f = mw == -INFINITY ? 0.f : expf(mw - M);
@@ -290,7 +293,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
 extern "C" int li_diff_attn(const void* q, void* out, int dt, void* k_pages, void* v_pages, int64_t page_stride,
                             const int* page_table, int max_pages, const int* pos, const int* tok_slot, int n, int H, int G,
                             int maps, int d, int dv, float scale, int block, int window, float lambda, float out_eps,
-                            float out_scale, hipStream_t stream) {
+                            float out_scale, const float* sink, hipStream_t stream) {
     if (n <= 0) return LI_OK;
     if (H <= 0 || G <= 0 || H % G || d <= 0 || dv <= 0 || block < 0 || window < 0) return LI_BAD_ARG;
     if (maps < 1 || maps > 2 || dv > 64 * DA_MAXV) return LI_UNSUPPORTED;
@@ -299,7 +302,7 @@ extern "C" int li_diff_attn(const void* q, void* out, int dt, void* k_pages, voi
     const size_t lds = (size_t)(maps * round_up(d, 16) + 2 * DA_WAVES * maps + DA_WAVES * maps * dv) * sizeof(float);
     if (lds > 60000) return LI_UNSUPPORTED;
 #define GO(M) diff_attn_kernel<T, M><<<grid, blk, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, H, G, d, dv, scale, \
-                                                                 block, window, lambda, out_eps, out_scale)
+                                                                 block, window, lambda, out_eps, out_scale, sink)
     DISPATCH_T(dt, { if (maps == 1) GO(1); else GO(2); });
 #undef GO
     LI_CHECK_LAUNCH();
@@ -316,9 +319,10 @@ extern "C" int li_diff_attn(const void* q, void* out, int dt, void* k_pages, voi
 // ---------------------------------------------------------------------------
 #define CONV_MAX_TAPS 16
 
+template <class T, bool SILU, bool ADD>
 __global__ void conv_silu_kernel(const float* __restrict__ in, int stride, int col0, const float* __restrict__ w,
                                  const float* __restrict__ b, const float* __restrict__ hist, const int* __restrict__ pos,
-                                 const int* __restrict__ tok_slot, float* __restrict__ out, int channels, int taps) {
+                                 const int* __restrict__ tok_slot, T* __restrict__ out, int channels, int taps) {
     const int t = blockIdx.x, p = pos[t], slot = tok_slot[t];
     // how many tokens before this one its sequence has in this step (at most taps - 1 matter)
     int inside = 0;
@@ -332,7 +336,8 @@ __global__ void conv_silu_kernel(const float* __restrict__ in, int stride, int c
             else if (p - back >= 0) u = h[(int64_t)(taps - 1 - (back - inside)) * channels + c];
             acc += w[(int64_t)c * taps + (taps - 1 - back)] * u;
         }
-        out[(int64_t)t * channels + c] = siluf_(acc);
+        if (ADD) acc += in[(int64_t)t * stride + col0 + c];        // the input itself beside its convolution
+        out[(int64_t)t * channels + c] = from_f32<T>(SILU ? siluf_(acc) : acc);
     }
 }
 
@@ -359,7 +364,26 @@ extern "C" int li_conv_silu(const float* in, int stride, int col0, const float* 
     if (n_tokens <= 0) return LI_OK;
     if (channels <= 0 || taps < 1 || taps > CONV_MAX_TAPS) return LI_BAD_ARG;
     dim3 cgrid(n_tokens, (channels + 255) / 256);
-    conv_silu_kernel<<<cgrid, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, out, channels, taps);
+    conv_silu_kernel<float, true, false><<<cgrid, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, out, channels, taps);
+    if (taps > 1) {
+        dim3 grid(n_seqs, (channels + 255) / 256);
+        conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);
+    }
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// The same convolution without an activation, the input added to it: out = u + conv(u), in type dt (what a mixer
+// reads when its input first passes a short convolution over time).
+extern "C" int li_conv_add(const float* in, int stride, int col0, const float* w, const float* b, float* hist,
+                           const int* pos, const int* tok_slot, const int* seq_slot, const int* seq_qstart,
+                           const int* seq_qlen, void* out, int dt, int n_tokens, int n_seqs, int channels, int taps,
+                           hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (channels <= 0 || taps < 1 || taps > CONV_MAX_TAPS) return LI_BAD_ARG;
+    dim3 cgrid(n_tokens, (channels + 255) / 256);
+    DISPATCH_T(dt, (conv_silu_kernel<T, false, true><<<cgrid, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, (T*)out,
+                                                                                channels, taps)));
     if (taps > 1) {
         dim3 grid(n_seqs, (channels + 255) / 256);
         conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);
@@ -623,13 +647,15 @@ extern "C" int li_small_logits(const void* h, int dt, const float* w, float* out
 // s / (sum of the chosen s + 1e-20) * route_scale.  The first n_real outputs are experts with matrices: their
 // weights (0 where not chosen) go to `weights` [T, n_real (+ 1)], the gate's sigmoid into the last column.  The
 // outputs behind them pass the token's input on: residual[t] += (sum of their weights) * h[t].
+// `sigmoid_scores`: s = sigmoid of every output's logit instead of the softmax.  `renorm` 0: a chosen output's weight
+// is its own s * route_scale, not divided by the sum of the chosen.
 // ---------------------------------------------------------------------------
 template <class T>
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int n_cols,
                                                        const float* __restrict__ correction, const T* __restrict__ h,
                                                        float* __restrict__ residual, float* __restrict__ weights,
                                                        int width, int n_route, int n_real, int top, int has_gate,
-                                                       float route_scale) {
+                                                       float route_scale, int sigmoid_scores, int renorm) {
     extern __shared__ float lds[];
     float* s = lds;                      // [n_route] softmax scores
     float* c = s + n_route;              // [n_route] choice scores, -inf once chosen
@@ -641,6 +667,10 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     float sum = 0.f;
     for (int i = lane; i < n_route; i += 64) { const float e = expf(z[i] - mx); s[i] = e; sum += e; }
     sum = wave_sum(sum);
+    if (sigmoid_scores) {
+        sum = 1.f;
+        for (int i = lane; i < n_route; i += 64) s[i] = sigmoidf_(z[i]);
+    }
     const int wcols = n_real + (has_gate ? 1 : 0);
     for (int i = lane; i < n_route; i += 64) {
         s[i] /= sum;
@@ -661,7 +691,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
         if (lane == 0) c[bi] = -INFINITY;
         __syncthreads();
     }
-    const float f = route_scale / (chosen_sum + 1e-20f);
+    const float f = renorm ? route_scale / (chosen_sum + 1e-20f) : route_scale;
     float pass = 0.f;                    // the weight of the outputs that pass the input on
     // every lane knows the chosen set through c == -inf
     for (int i = lane; i < n_route; i += 64) {
@@ -678,7 +708,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
 
 extern "C" int li_moe_route(const float* logits, int n_cols, const float* correction, const void* h, int dt,
                             float* residual, float* weights, int n, int width, int n_route, int n_real, int top,
-                            int has_gate, float route_scale, hipStream_t stream) {
+                            int has_gate, float route_scale, int sigmoid_scores, int renorm, hipStream_t stream) {
     if (n <= 0) return LI_OK;
     if (n_route <= 0 || n_real < 0 || n_real > n_route || top < 1 || top > n_route || n_cols < n_route + (has_gate == 1 ? 1 : 0) ||
         has_gate < 0 || has_gate > 2)
@@ -686,7 +716,8 @@ extern "C" int li_moe_route(const float* logits, int n_cols, const float* correc
     if (n_route > 4096) return LI_UNSUPPORTED;
     const size_t lds = (size_t)2 * n_route * sizeof(float);
     DISPATCH_T(dt, (moe_route_kernel<T><<<n, 64, lds, stream>>>(logits, n_cols, correction, (const T*)h, residual, weights,
-                                                                 width, n_route, n_real, top, has_gate, route_scale)));
+                                                                 width, n_route, n_real, top, has_gate, route_scale,
+                                                                 sigmoid_scores, renorm)));
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
@@ -772,7 +803,7 @@ __global__ void scatter_add_rows_kernel(float* __restrict__ residual, const floa
                                         const int* __restrict__ idx, const float* __restrict__ weights, int wcols, int col,
                                         int width) {
     const int64_t r = blockIdx.x, dst = idx ? idx[r] : r;
-    const float w = weights[dst * wcols + col];
+    const float w = col >= 0 ? weights[dst * wcols + col] : 1.f;        // col < 0: the rows are added as they are
     for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x)
         residual[dst * width + i] += w * y[r * width + i];
 }
@@ -780,7 +811,7 @@ __global__ void scatter_add_rows_kernel(float* __restrict__ residual, const floa
 extern "C" int li_scatter_add_rows(float* residual, const float* y, const int* idx, const float* weights, int wcols,
                                    int col, int n, int width, hipStream_t stream) {
     if (n <= 0) return LI_OK;
-    if (width <= 0 || col < 0 || col >= wcols) return LI_BAD_ARG;
+    if (width <= 0 || col >= wcols) return LI_BAD_ARG;
     dim3 grid(n, n >= 1024 ? 1 : (width + 1023) / 1024);
     scatter_add_rows_kernel<<<grid, 256, 0, stream>>>(residual, y, idx, weights, wcols, col, width);
     LI_CHECK_LAUNCH();

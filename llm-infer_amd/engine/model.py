@@ -49,6 +49,15 @@ class DecoderModel(Part):
             if key is not None and key not in self.stream_parts:
                 self.stream_parts[key] = _make("stream", b, dtype, dev)
             self._before.append(key)
+        # parts that form the stream's next value from all its values so far, after a run of a layer
+        self._after = []
+        for e in spec.schedule:
+            a = getattr(e, "after", None)
+            key = None if a is None else ("after", a.kind, a.prefix, repr(sorted(a.params.items())))
+            if key is not None and key not in self.stream_parts:
+                self.stream_parts[key] = _make("stream", a, dtype, dev)
+            self._after.append(key)
+        self._n_after = sum(k is not None for k in self._after)
         self.final_norm = _make("norm", spec.final_norm, dtype, dev)
         self.head = _make("head", spec.head, dtype, dev)
         self.schedule = list(spec.schedule)
@@ -65,6 +74,8 @@ class DecoderModel(Part):
             for k, count in enumerate(self._asks[e.layer]):
                 self._unit[i, k] = list(range(n, n + count))
                 n += count
+        # an embedding may keep state of every sequence too (the token before, say): its units come last
+        self._embedding_units = list(range(n, n + len(self._embedding_specs())))
         self._table = collect_params(self)
 
     def _position(self, spec, dtype, dev):
@@ -124,20 +135,34 @@ class DecoderModel(Part):
             stack += list(part.children())
 
     # -- cache -------------------------------------------------------------
+    def _embedding_specs(self) -> list:
+        return list(self.embedding.cache_specs()) if hasattr(self.embedding, "cache_specs") else []
+
     def cache_specs(self) -> list:
-        """For each unit (each mixer of each schedule entry, in order) what it asks of the cache
-        (None: it reads another's)."""
+        """For each unit (each mixer of each schedule entry, in order, then whatever the embedding keeps of every
+        sequence) what it asks of the cache (None: it reads another's)."""
         return [None if e.cache_from is not None else spec
-                for e in self.schedule for m in self.layer_mixers[e.layer] for spec in cache_specs_of(m)]
+                for e in self.schedule for m in self.layer_mixers[e.layer] for spec in cache_specs_of(m)] + self._embedding_specs()
 
     # -- the forward pass of one step ---------------------------------------
     def forward(self, ctx, cache) -> torch.Tensor:
         """Runs the step's tokens through the schedule; returns float32 logits [n_want, vocab]."""
-        x = x0 = self.embedding.forward(ctx)
+        if self._embedding_units:
+            x = x0 = self.embedding.forward(ctx, [cache.view(u) for u in self._embedding_units])
+        else:
+            x = x0 = self.embedding.forward(ctx)
+        history, n_hist = None, 0
+        if self._n_after:
+            # the stream's values side by side: the embedding's output, then the result of every run that an
+            # ``after`` part follows (the run works in place on the row that the part before it has written)
+            history = torch.empty((self._n_after + 2,) + tuple(x0.shape), dtype=torch.float32, device=x0.device)
+            history[0].copy_(x0)
+            history[1].copy_(x0)
+            x, n_hist = history[1], 1
         for i, e in enumerate(self.schedule):
             if self._before[i] is not None:
                 x = self.stream_parts[self._before[i]].forward(x, x0, ctx)       # a new tensor: x0 stays as it is
-            elif x is x0 and self.stream_parts:
+            elif x is x0 and self.stream_parts and history is None:
                 x = ops.copy_rows(x0)            # the layers add in place, and a later part reads the embedding's output
             owner = i if e.cache_from is None else e.cache_from
             # one view for a mixer, or the list of its views for one that asks several things of the cache
@@ -151,6 +176,9 @@ class DecoderModel(Part):
                 layer.forward(x, ctx, views, e.cache_from is None, next_norm=first() if first else None)
             else:
                 layer.forward(x, ctx, views, e.cache_from is None)
+            if self._after[i] is not None:
+                n_hist += 1                      # x is history[n_hist - 1], now a finished value of the stream
+                x = self.stream_parts[self._after[i]].forward_after(history, n_hist, history[n_hist], ctx)
         if ctx.n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         h = self.final_norm.forward(x, ctx.want_rows)

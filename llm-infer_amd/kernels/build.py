@@ -191,12 +191,14 @@ def mixers_library(force=False):
     return _load("libli_mixers.so", MIXER_SOURCES, (), force)
 
 
-HYBRID_SOURCES = ("hybrid.hip",)
+HYBRID_SOURCES = ("hybrid.hip", "latent.hip")
 
 
 def hybrid_library(force=False):
     """The kernels of hybrid decoders (csrc/hybrid.hip: differential attention over blocks of positions, the
-    state-space recurrence and its convolution, the experts' router): a library of its own, as the mixers' is."""
+    state-space recurrence and its convolution, the experts' router; csrc/latent.hip: latent attention's
+    preparation and products per head, the matrix-memory recurrence, the bigram embedding, the depth-weighted
+    average of the residual stream): a library of its own, as the mixers' is."""
     return _load("libli_hybrid.so", HYBRID_SOURCES, (), force)
 
 

@@ -1113,7 +1113,7 @@ def polynorm(z, coef, eps, out_dtype) -> torch.Tensor:
 # routed experts, a scaled embedding with sinusoidal positions
 # ---------------------------------------------------------------------------
 _hybrid = None
-ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu2": 3}
 
 
 def hybrid():
@@ -1153,9 +1153,9 @@ def concat_cast(a, b, dtype) -> torch.Tensor:
 
 
 def activation(z, kind: str, out_dtype) -> torch.Tensor:
-    """act(z) for float32 z in ``out_dtype``; kind: gelu (erf), gelu_tanh, silu."""
+    """act(z) for float32 z in ``out_dtype``; kind: gelu (erf), gelu_tanh, silu, relu2 (the square of relu)."""
     _dev(z)
-    _need(z.dtype == torch.float32 and kind in ACTIVATIONS and out_dtype in DT, f"activation {kind!r}: float32 in, gelu/gelu_tanh/silu")
+    _need(z.dtype == torch.float32 and kind in ACTIVATIONS and out_dtype in DT, f"activation {kind!r}: float32 in, one of {', '.join(ACTIVATIONS)}")
     out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
     _check(hybrid().li_activation(_ptr(z), _ptr(out), DT[out_dtype], c_int64(z.numel()), ACTIVATIONS[kind], _stream()),
            "activation")
@@ -1253,17 +1253,19 @@ def diff_tiles(ctx, block=None, window=None):
 
 
 def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale, block, window, lam, out_eps, out_scale,
-                   out_dtype, tiles=None) -> torch.Tensor:
+                   out_dtype, tiles=None, sink=None) -> torch.Tensor:
     """Attention of ``maps`` softmax maps (1 or 2) over the same values: o = a_1 - lam a_2, then (``out_eps`` not
     None) o divided by its root mean square over dv, times ``out_scale``.  A token at position p sees the keys
     from p - p % block on (``block`` 0: from 0; ``window`` w: at most the last w).  q [T, H, maps * DP] as
     ``qk_norm_store`` leaves it; returns [T, H * dv] in ``out_dtype``, the cache's type.  A float32 cache runs one
     workgroup per (token, head); a 16-bit cache runs on the matrix cores, one wave per (pair of tiles, head) with
-    ``tiles`` from ``diff_tiles`` for the same block and window (None: every token an item of its own)."""
-    _dev(q, pos, tok_slot)
+    ``tiles`` from ``diff_tiles`` for the same block and window (None: every token an item of its own).
+    ``sink`` (float32 [H]): every map's sum of weights also counts exp(sink[head]), which has no key and no value."""
+    _dev(q, pos, tok_slot, sink)
+    _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == n_heads), "sink: float32 [H]")
     t = q.shape[0]
     dp = padded_map_dim(d)
-    _need(maps in (1, 2) and dv <= 256 and n_heads % n_kv_heads == 0, "diff_attention: one or two maps, values up to 256 wide")
+    _need(maps in (1, 2) and dv <= 512 and n_heads % n_kv_heads == 0, "diff_attention: one or two maps, values up to 512 wide")
     _i32(pos, t, "positions")
     _i32(tok_slot, t, "slots")
     k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, n_kv_heads, maps * dp, dv)
@@ -1271,13 +1273,13 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
     _need(out_dtype == k_pages.dtype, "diff_attention: the output has the cache's type")
     out = torch.empty((t, n_heads * dv), dtype=out_dtype, device=q.device)
     tail = (c_float(scale), int(block or 0), int(window or 0), c_float(lam), c_float(-1.0 if out_eps is None else out_eps),
-            c_float(out_scale), _stream())
-    if out_dtype == torch.float32:
+            c_float(out_scale), _ptr(sink), _stream())
+    if out_dtype == torch.float32 or not diff_attention_fits(d, dv):
+        # (also a 16-bit cache whose sizes the matrix-core kernel does not take)
         _check(hybrid().li_diff_attn(_ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride),
                                      _ptr(page_table), page_table.shape[1], _ptr(pos), _ptr(tok_slot), t, n_heads, n_kv_heads,
                                      maps, d, dv, *tail), "diff_attn")
         return out
-    _need(dp <= 256, "diff_attention on the matrix cores: a map's keys up to 256 wide")
     tile_t0, tile_n, n_tiles = tiles if tiles is not None else (None, None, t)
     if tiles is not None:
         _i32(tile_t0, 2 * n_tiles, "tile starts")
@@ -1287,6 +1289,11 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
         page_table.shape[1], _ptr(pos), _ptr(tok_slot), _ptr(tile_t0), _ptr(tile_n), n_tiles, n_heads, n_kv_heads, maps, dv,
         *tail), "diffattn")
     return out
+
+
+def diff_attention_fits(d: int, dv: int) -> bool:
+    """True if the matrix-core kernel takes a map's keys of size ``d`` and values of size ``dv``."""
+    return padded_map_dim(d) <= 256 and (dv + 31) // 32 * 32 <= 256
 
 
 def small_logits(h, w) -> torch.Tensor:
@@ -1402,12 +1409,14 @@ def gated_group_norm(y, zrows, z_col, weight, groups, eps, out_dtype) -> torch.T
     return out
 
 
-def moe_route(logits, correction, h, residual, n_route, n_real, top, has_gate, scale) -> torch.Tensor:
+def moe_route(logits, correction, h, residual, n_route, n_real, top, has_gate, scale, sigmoid_scores: bool = False,
+              renorm: bool = True) -> torch.Tensor:
     """Routing weights of every token: softmax over the first ``n_route`` columns of ``logits`` (float32), the ``top``
     largest of score + correction chosen, their scores divided by their sum (+ 1e-20) times ``scale``.  Returns
     float32 [T, n_real (+ 1)]: the weights of the first ``n_real`` outputs (0 where not chosen) and, with
     ``has_gate`` 1, sigmoid of the column behind the router's (2: the constant 1; 0: no such column).  The outputs from ``n_real`` on pass the token on:
-    residual[t] += (their weights' sum) * h[t]."""
+    residual[t] += (their weights' sum) * h[t].  ``sigmoid_scores``: the scores are the sigmoid of every output's logit
+    instead of the softmax; ``renorm`` False: a chosen output's weight is its own score times ``scale``."""
     _dev(logits, correction, h, residual)
     _f32_rows(logits, "router logits")
     t, width = h.shape
@@ -1419,7 +1428,8 @@ def moe_route(logits, correction, h, residual, n_route, n_real, top, has_gate, s
     _drop_row_stats(residual)
     w = torch.empty((t, n_real + int(bool(has_gate))), dtype=torch.float32, device=h.device)
     _check(hybrid().li_moe_route(_ptr(logits), logits.shape[1], _ptr(correction), _ptr(h), DT[h.dtype], _ptr(residual), _ptr(w),
-                                 t, width, n_route, n_real, top, has_gate, c_float(scale), _stream()), "moe_route")
+                                 t, width, n_route, n_real, top, has_gate, c_float(scale), int(bool(sigmoid_scores)),
+                                 int(bool(renorm)), _stream()), "moe_route")
     return w
 
 
@@ -1455,12 +1465,13 @@ def gather_rows(h, idx, n: int) -> torch.Tensor:
 
 
 def scatter_add_rows(residual, y, idx, weights, col: int) -> None:
-    """residual[idx[r]] += weights[idx[r]][col] * y[r] for every row of ``y`` (``idx`` None: row r itself); no row
-    may be named twice."""
+    """residual[idx[r]] += weights[idx[r]][col] * y[r] for every row of ``y`` (``idx`` None: row r itself; ``col`` None:
+    the rows are added as they are); no row may be named twice."""
     _dev(residual, y, idx, weights)
     n, width = y.shape
     _need(residual.dtype == torch.float32 and y.dtype == torch.float32 and residual.shape[1] == width, "scatter_add_rows: float32 rows of one width")
-    _need(weights.dtype == torch.float32 and weights.dim() == 2 and weights.shape[0] == residual.shape[0] and 0 <= col < weights.shape[1],
+    col = -1 if col is None else col
+    _need(weights.dtype == torch.float32 and weights.dim() == 2 and weights.shape[0] == residual.shape[0] and -1 <= col < weights.shape[1],
           "scatter_add_rows: a weight for every row of the residual")
     _need(idx is None and n == residual.shape[0] or idx is not None and idx.dtype == torch.int32 and idx.numel() >= n,
           "scatter_add_rows: int32 indices for every row of y")
@@ -1472,3 +1483,205 @@ def scatter_add_rows(residual, y, idx, weights, col: int) -> None:
 def copy_rows(x: torch.Tensor) -> torch.Tensor:
     """A copy of ``x`` in memory of its own (one device-to-device copy on the current stream)."""
     return x.clone()
+
+
+# ---------------------------------------------------------------------------
+# latent attention, the matrix-memory recurrence, a bigram embedding, the depth-weighted residual stream
+# (csrc/latent.hip, in the hybrid library)
+# ---------------------------------------------------------------------------
+def _seq_arrays(ctx, n_tokens):
+    """(seq_slot, seq_qstart, seq_qlen) of a step; the last two None for a step of one token a sequence."""
+    _i32(ctx.seq_slot, ctx.n_seqs, "sequence slots")
+    qstart, qlen = getattr(ctx, "seq_qstart", None), getattr(ctx, "seq_qlen", None)
+    _need((qstart is None) == (qlen is None) and (qstart is not None or n_tokens == ctx.n_seqs),
+          "per-sequence starts and lengths, or one token a sequence")
+    return ctx.seq_slot, qstart, qlen
+
+
+def embed_bigram(table, bigram, ctx, prev_state, scale: float, mul_prev: int, mul_cur: int, out=None) -> torch.Tensor:
+    """x[t] = table[token] * scale + bigram[(previous token * mul_prev + token * mul_cur) mod buckets], buckets =
+    rows of ``bigram`` - 1; a sequence's first token takes the last row.  ``prev_state`` int32 [slots]: the token
+    before the first one that a sequence brings to this step; left at the sequence's last token of the step."""
+    _dev(table, bigram, prev_state, out)
+    n, (vocab, d) = ctx.n_tokens, table.shape
+    _need(table.dim() == 2 and bigram.dim() == 2 and bigram.shape[1] == d and bigram.shape[0] >= 2 and table.dtype == bigram.dtype
+          and table.dtype in DT, "embed_bigram: two float tables of one width and type")
+    _i32(ctx.token_ids, n, "tokens")
+    _i32(ctx.pos, n, "positions")
+    _i32(ctx.tok_slot, n, "slots")
+    _need(prev_state.dtype == torch.int32 and prev_state.dim() == 1, "embed_bigram: int32 [slots] previous tokens")
+    seq_slot, qstart, qlen = _seq_arrays(ctx, n)
+    if out is None:
+        out = torch.empty((n, d), dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.shape == (n, d), "embed_bigram out: float32 [T, d]")
+    _drop_row_stats(out)
+    _check(hybrid().li_embed_bigram(_ptr(table), _ptr(bigram), DT[table.dtype], _ptr(ctx.token_ids), _ptr(ctx.pos),
+                                    _ptr(ctx.tok_slot), _ptr(seq_slot), _ptr(qstart), _ptr(qlen), _ptr(prev_state), _ptr(out), n,
+                                    ctx.n_seqs, d, c_float(scale), c_int64(mul_prev), c_int64(mul_cur), bigram.shape[0] - 1,
+                                    _stream()), "embed_bigram")
+    return out
+
+
+def depth_average(history: torch.Tensor, n: int, weights: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = sum over j < n of weights[j] * history[j]; ``history`` float32 [runs, T, width], ``out`` float32 [T, width]
+    (it may be a later row of ``history``)."""
+    _dev(history, weights, out)
+    _need(history.dtype == torch.float32 and history.dim() == 3 and 1 <= n <= history.shape[0], "depth_average: float32 [runs, T, width]")
+    _need(weights.dtype == torch.float32 and weights.numel() >= n, "depth_average: a float32 weight for every term")
+    _need(out.dtype == torch.float32 and tuple(out.shape) == tuple(history.shape[1:]), "depth_average out: float32 [T, width]")
+    _drop_row_stats(out)
+    _check(hybrid().li_depth_average(_ptr(history), c_int64(history.stride(0)), _ptr(weights), n, _ptr(out), c_int64(out.numel()),
+                                     _stream()), "depth_average")
+    return out
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap) in place (float32)."""
+    _dev(x)
+    _need(x.dtype == torch.float32 and cap > 0, "softcap: float32 values, a positive cap")
+    _check(hybrid().li_softcap(_ptr(x), c_int64(x.numel()), c_float(cap), _stream()), "softcap")
+    return x
+
+
+def conv_add(rows, weight, history, ctx, out_dtype) -> torch.Tensor:
+    """u + conv(u) for the float32 ``rows`` u [T, channels]: a causal convolution per channel over time, weight
+    float32 [channels, taps] (last column: the current token), no bias, no activation; ``history`` float32
+    [slots, taps - 1, channels] holds every sequence's last inputs and is brought up to date.  Returns ``out_dtype``."""
+    _dev(rows, weight, history)
+    _f32_rows(rows, "conv rows")
+    t, channels = rows.shape
+    taps = weight.shape[1]
+    _need(weight.dtype == torch.float32 and weight.shape == (channels, taps) and 1 <= taps <= 16, "conv weight: float32 [channels, taps <= 16]")
+    _need(history.dtype == torch.float32 and history.dim() == 3 and tuple(history.shape[1:]) == (max(taps - 1, 1), channels),
+          "conv history: float32 [slots, taps - 1, channels]")
+    _i32(ctx.pos, t, "positions")
+    _i32(ctx.tok_slot, t, "slots")
+    seq_slot, qstart, qlen = _seq_arrays(ctx, t)
+    out = torch.empty((t, channels), dtype=out_dtype, device=rows.device)
+    _check(hybrid().li_conv_add(_ptr(rows), channels, 0, _ptr(weight), None, _ptr(history), _ptr(ctx.pos), _ptr(ctx.tok_slot),
+                                _ptr(seq_slot), _ptr(qstart), _ptr(qlen), _ptr(out), DT[out_dtype], t, ctx.n_seqs, channels, taps,
+                                _stream()), "conv_add")
+    return out
+
+
+def latent_store(proj, q_col, kv_col, norm_weight, eps, inv_freq, rot, pos, tok_slot, kv, n_heads, d, rd, r) -> torch.Tensor:
+    """From the float32 rows of latent attention's input product (from column ``q_col`` every head's [d unrotated | rd
+    rotated] query dimensions, from ``kv_col`` [latent r | rotated key part rd]): the latent divided by its root mean
+    square, times ``norm_weight`` [r]; the rotated parts turned by position (the first ``rot`` of their rd dimensions
+    in pairs (2i, 2i + 1), angle pos * inv_freq[i]); the key [latent | rotated part] (zeros up to the next multiple
+    of 16) and the value (the latent) into the pages.  Returns q [T, H, KW] in the cache's type with every head's
+    rotated part from column r on; the first r columns are left for ``head_linear``."""
+    _dev(proj, norm_weight, inv_freq, pos, tok_slot)
+    _f32_rows(proj, "latent_store rows")
+    t = proj.shape[0]
+    kw = padded_map_dim(r + rd)
+    _need(q_col >= 0 and kv_col >= 0 and max(q_col + n_heads * (d + rd), kv_col + r + rd) <= proj.shape[1], "latent_store: columns beyond the rows")
+    _need(norm_weight.dtype == torch.float32 and norm_weight.shape == (r,), "latent norm weight: float32 [r]")
+    _need(0 <= rot <= rd and rot % 2 == 0, "latent_store: an even number of rotated dimensions within rd")
+    if rot:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() >= rot // 2, "inv_freq: float32 [rot / 2]")
+    _i32(pos, t, "positions")
+    _i32(tok_slot, t, "slots")
+    k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, 1, kw, r)
+    q = torch.empty((t, n_heads, kw), dtype=k_pages.dtype, device=proj.device)
+    _check(hybrid().li_latent_store(_ptr(proj), proj.shape[1], q_col, kv_col, _ptr(norm_weight), c_float(eps), _ptr(inv_freq), rot,
+                                    _ptr(pos), _ptr(tok_slot), _ptr(q), _ptr(k_pages), _ptr(v_pages), c_int64(page_stride),
+                                    _ptr(page_table), page_table.shape[1], DT[k_pages.dtype], t, n_heads, d, rd, r, _stream()),
+           "latent_store")
+    return q
+
+
+def head_linear(x, x_col, x_head_stride, w, out, out_col, out_head_stride, gate=None, gate_col=0) -> torch.Tensor:
+    """A product per head: out[t, out_col + h * out_head_stride + j] = sum over i of w[h, i, j] * x[t, x_col + h *
+    x_head_stride + i], ``w`` [H, n_in, n_out] in the model's type, ``x`` [T, ...] float32 or of that type, ``out``
+    [T, ...] of that type (both may be wider rows in which a head's part lies).  ``gate`` (float32 rows): the result
+    is multiplied by sigmoid(gate[t, gate_col + h * n_out + j]).  Sums are float32."""
+    _dev(x, w, out, gate)
+    x2, o2 = x.view(x.shape[0], -1), out.view(out.shape[0], -1)
+    t = x2.shape[0]
+    _need(w.dim() == 3 and w.dtype in DT and x2.dtype in (torch.float32, w.dtype) and o2.dtype == w.dtype and o2.shape[0] == t,
+          "head_linear: weights [H, n_in, n_out], rows of their type (or float32 in)")
+    H, n_in, n_out = w.shape
+    _need(x_col >= 0 and x_col + (H - 1) * x_head_stride + n_in <= x2.shape[1], "head_linear: input columns beyond the rows")
+    _need(out_col >= 0 and out_col + (H - 1) * out_head_stride + n_out <= o2.shape[1], "head_linear: output columns beyond the rows")
+    if gate is not None:
+        _f32_rows(gate, "head_linear gate")
+        _need(gate.shape[0] == t and gate_col >= 0 and gate_col + H * n_out <= gate.shape[1], "head_linear: gate columns beyond the rows")
+    _need(n_in <= 960, "head_linear: up to 960 inputs a head")
+    _drop_row_stats(out)
+    _check(hybrid().li_head_linear(c_void_p(x2.data_ptr() + x_col * x2.element_size()), DT[x2.dtype], c_int64(x2.shape[1]),
+                                   x_head_stride, _ptr(w), DT[w.dtype], c_void_p(o2.data_ptr() + out_col * o2.element_size()),
+                                   c_int64(o2.shape[1]), out_head_stride,
+                                   c_void_p(gate.data_ptr() + 4 * gate_col) if gate is not None else None,
+                                   c_int64(gate.shape[1] if gate is not None else 0), t, H, n_in, n_out, _stream()), "head_linear")
+    return out
+
+
+def mlstm_scan(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, q_scale, state, norm_state, ctx, heads, d, dv) -> torch.Tensor:
+    """The matrix-memory recurrence in float32 over the tokens of a step.  q, k [heads, d], v [heads, dv] and the two raw
+    gates [heads] are columns of the float32 rows ``proj``; with i = cap tanh((gi + i_bias) / cap), f = logsigmoid(cap
+    tanh((gf + f_bias) / cap)):  m <- max(f + m, i);  S <- exp(f + m_old - m) S + exp(i - m) k v^T, n likewise with k;
+    y = S^T q / (max(|n . q|, exp(-m)) + 1e-6), q times ``q_scale``.  ``state`` float32 [slots, heads, d, dv] and
+    ``norm_state`` float32 [slots, heads, d + 1] (n, then m) are read and left up to date.  Returns y float32 [T, heads * dv]."""
+    _dev(proj, i_bias, f_bias, state, norm_state)
+    _f32_rows(proj, "mlstm projections")
+    t = proj.shape[0]
+    _need(1 <= d <= 256 and dv >= 1 and cap > 0, "mlstm: keys up to 256 wide, a positive cap")
+    _need(max(q_col + heads * d, k_col + heads * d, v_col + heads * dv, i_col + heads, f_col + heads) <= proj.shape[1]
+          and min(q_col, k_col, v_col, i_col, f_col) >= 0, "mlstm: columns beyond the rows")
+    for b in (i_bias, f_bias):
+        _need(b is None or (b.dtype == torch.float32 and b.shape == (heads,)), "mlstm: float32 [heads] gate biases")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, d, dv), "mlstm state: float32 [slots, heads, d, dv]")
+    _need(norm_state.dtype == torch.float32 and tuple(norm_state.shape[1:]) == (heads, d + 1) and norm_state.shape[0] == state.shape[0],
+          "mlstm normaliser state: float32 [slots, heads, d + 1]")
+    seq_slot, qstart, qlen = _seq_arrays(ctx, t)
+    y = torch.empty((t, heads * dv), dtype=torch.float32, device=proj.device)
+    fresh = torch.empty((ctx.n_seqs, heads, d + 1), dtype=torch.float32, device=proj.device)
+    _check(hybrid().li_mlstm_scan(_ptr(proj), proj.shape[1], q_col, k_col, v_col, i_col, f_col, _ptr(i_bias), _ptr(f_bias),
+                                  c_float(cap), c_float(q_scale), _ptr(state), _ptr(norm_state), _ptr(fresh), _ptr(seq_slot),
+                                  _ptr(qstart), _ptr(qlen), _ptr(y), ctx.n_seqs, heads, d, dv, _stream()), "mlstm_scan")
+    return y
+
+
+def gated_head_norm(y, weight, gate_rows, gate_col, heads, eps, out_dtype) -> torch.Tensor:
+    """Every head's part of a float32 row [heads * dv] divided by its own root mean square, then times ``weight``
+    [heads * dv] (None: none) and sigmoid of columns gate_col .. of the float32 ``gate_rows`` (None: no gate)."""
+    _dev(y, weight, gate_rows)
+    _f32_rows(y, "head norm rows")
+    t, n = y.shape
+    _need(heads >= 1 and n % heads == 0, "head norm: equal heads")
+    _need(weight is None or (weight.dtype == torch.float32 and weight.shape == (n,)), "head norm weight: float32 [heads * dv]")
+    if gate_rows is not None:
+        _f32_rows(gate_rows, "head norm gate")
+        _need(gate_rows.shape[0] == t and gate_col >= 0 and gate_col + n <= gate_rows.shape[1], "head norm: gate columns beyond the rows")
+    out = torch.empty((t, n), dtype=out_dtype, device=y.device)
+    _check(hybrid().li_gated_head_norm(_ptr(y), _ptr(weight),
+                                       c_void_p(gate_rows.data_ptr() + 4 * gate_col) if gate_rows is not None else None,
+                                       c_int64(gate_rows.shape[1] if gate_rows is not None else 0), _ptr(out), DT[out_dtype], t,
+                                       heads, n // heads, c_float(eps), _stream()), "gated_head_norm")
+    return out
+
+
+def expert_act(z, weights, n_blocks, ff, tail, kind: str, on_input: bool, out_dtype, idx=None, col=None) -> torch.Tensor:
+    """The hidden rows of experts side by side (``z`` float32 [rows, n_blocks * ff + tail], the sums of the up
+    products) through the activation ``kind`` with the routing weight: block e of row r takes weights[r][e], the
+    tail weights[r][n_blocks]; ``idx`` (int32): row r of ``z`` is token idx[r]; ``col``: every block takes that
+    column (the rows of one expert).  ``on_input``: act(weight * z), the weight on the expert's input; else weight *
+    act(z).  ``weights`` None: the plain activation."""
+    _dev(z, weights, idx)
+    _f32_rows(z, "expert rows")
+    rows = z.shape[0]
+    _need(kind in ACTIVATIONS and z.shape[1] == n_blocks * ff + tail, "expert_act: [rows, blocks * ff + tail], a known activation")
+    wcols = 0
+    if weights is not None:
+        _need(weights.dtype == torch.float32 and weights.dim() == 2, "expert_act: float32 weights [tokens, columns]")
+        wcols = weights.shape[1]
+        _need(wcols >= (n_blocks + int(tail > 0) if col is None else col + 1), "expert_act: a weight for every block")
+        if idx is None:
+            _need(weights.shape[0] == rows, "expert_act: a row of weights for every row")
+        else:
+            _i32(idx, rows, "expert_act rows' tokens")
+    out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+    _check(hybrid().li_expert_act(_ptr(z), _ptr(weights), wcols, _ptr(idx), -1 if col is None else col, _ptr(out), DT[out_dtype],
+                                  rows, n_blocks, ff, tail, ACTIVATIONS[kind], int(bool(on_input)), _stream()), "expert_act")
+    return out

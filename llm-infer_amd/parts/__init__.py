@@ -9,11 +9,15 @@ from .sigmoid_attention import SigmoidAttention
 from .decay_attention import DecayLinearAttention
 from .diff_attention import DifferentialAttention
 from .state_space import SelectiveStateSpace
-from .stream import Reinject
-from .embedding import Embedding, LMHead
-from .block import Block, PostNormBlock, PreNormBlock, SubLayer
+from .stream import DepthAverage, Reinject
+from .embedding import BigramEmbedding, Embedding, LMHead
+from .block import Block, ParallelBlock, PostNormBlock, PreNormBlock, SubLayer
+from .short_conv import ConvMixer
+from .latent_attention import LatentAttention
+from .mlstm import MatrixLSTM
 
 __all__ = ["Part", "collect_params", "RMSNorm", "RotaryPosition", "NoPosition", "Attention", "GatedMLP",
            "Embedding", "LMHead", "Block", "PreNormBlock", "SubLayer", "LayerNorm", "PolyNormMLP", "ShiftedMixer",
            "ParallelMixers", "SigmoidAttention", "DecayLinearAttention", "PostNormBlock", "DifferentialAttention",
-           "SelectiveStateSpace", "Reinject", "DenseMLP", "RoutedExperts"]
+           "SelectiveStateSpace", "Reinject", "DenseMLP", "RoutedExperts", "DepthAverage", "BigramEmbedding", "ParallelBlock",
+           "ConvMixer", "LatentAttention", "MatrixLSTM"]

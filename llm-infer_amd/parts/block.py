@@ -93,6 +93,30 @@ class PreNormBlock(Block):
                 s.part.forward(h, x)
 
 
+@register_block("parallel")
+class ParallelBlock(Block):
+    """x <- x + sum over the sub-layers of part(norm(x)): every sub-layer reads the same x through a norm of its own,
+    and their results are added to it together.  All norms are taken before any part adds into the rows.  A part
+    that says ``reads_float32`` is handed its normed rows in float32 (a convolution over time ahead of a mixer, say)."""
+
+    def __init__(self, sublayers):
+        super().__init__(sublayers)
+        for s in self.sublayers:
+            if s.norm is None or s.post_norm is not None:
+                raise ValueError("a parallel block has one norm before each part and none after it")
+
+    def forward(self, x, ctx, cache_views, owns_cache=True):
+        views = iter(cache_views)
+        ops.expect_norm(x, None)                 # the rows are complete only after the last part: no norm rides along
+        normed = [s.norm.forward(x, out_dtype=torch.float32) if getattr(s.part, "reads_float32", False) else s.norm.forward(x)
+                  for s in self.sublayers]
+        for s, h in zip(self.sublayers, normed):
+            if s.role == "mixer":
+                s.part.forward(h, ctx, next(views), x, owns_cache)
+            else:
+                s.part.forward(h, x)
+
+
 @register_block("post_norm")
 class PostNormBlock(Block):
     """x <- norm(alpha * x + part(x)) for each sub-layer in turn: the parts read the residual stream itself and

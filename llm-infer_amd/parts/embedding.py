@@ -41,13 +41,52 @@ class Embedding(Part):
         return ops.embed_positions(self.weight, ctx.token_ids, ctx.pos, self.freq, self.scale)
 
 
+@register_embedding("bigram_embedding")
+class BigramEmbedding(Part):
+    """x = float32(table[token]) * ``scale`` + bigram[row]: beside the token's own row, a row of a second table chosen
+    by the token and the one before it, row = (previous * ``mul_prev`` + token * ``mul_cur``) mod ``buckets``; a
+    sequence's first token takes row number ``buckets``, the last of the table's buckets + 1 rows.
+
+    The token before the first one that a sequence brings to a step is state of the sequence: one int32 for every
+    slot (``StateSpec``), which the engine's cache keeps as it keeps a mixer's state, so prompts may be cut anywhere
+    and recorded decode steps feed it on the device.  ``names``: local names of the two tables."""
+
+    def __init__(self, *, vocab_size, hidden_size, buckets, mul_prev, mul_cur, scale=1.0, names=None, prefix, dtype, device):
+        if buckets < 1:
+            raise ValueError("bigram embedding: at least one bucket")
+        self.vocab_size, self.hidden_size, self.buckets = vocab_size, hidden_size, int(buckets)
+        self.mul_prev, self.mul_cur, self.scale = int(mul_prev), int(mul_cur), float(scale)
+        self.names = {"table": "weight", "bigram": "bigram", **(names or {})}
+        self.prefix, self.dtype, self.device = prefix, dtype, device
+        self.weight = self.bigram = None
+
+    def params(self):
+        return {self.names["table"]: ParamSpec((self.vocab_size, self.hidden_size)),
+                self.names["bigram"]: ParamSpec((self.buckets + 1, self.hidden_size))}
+
+    def bind(self, tensors):
+        self.weight, self.bigram = tensors[self.names["table"]], tensors[self.names["bigram"]]
+
+    def cache_specs(self):
+        from ..cache.specs import StateSpec
+        return [StateSpec((), "int32")]
+
+    def forward(self, ctx, views):
+        """``views``: the cache's views for ``cache_specs()``; float32 [T, hidden]."""
+        return ops.embed_bigram(self.weight, self.bigram, ctx, views[0].state, self.scale, self.mul_prev, self.mul_cur)
+
+
 @register_head("lm_head")
 class LMHead(Part):
     """logits = h W^T in float32 (src/model/model.cpp:93-98).  ``tied``: W is the embedding
     table (the reference has no tied models: it requires output.weight, model.cpp:35-38)."""
 
-    def __init__(self, *, vocab_size, hidden_size, tied, name="weight", prefix, dtype, device):
+    def __init__(self, *, vocab_size, hidden_size, tied, name="weight", softcap=None, prefix, dtype, device):
+        """``softcap`` c: the logits become c * tanh(logits / c)."""
         self.vocab_size, self.hidden_size, self.tied, self.name = vocab_size, hidden_size, tied, name
+        self.softcap = None if softcap is None else float(softcap)
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError("lm_head: a positive soft cap")
         self.prefix, self.dtype, self.device = prefix, dtype, device
         self.weight = None
 
@@ -66,4 +105,5 @@ class LMHead(Part):
         self.weight = ops.prepare_weight(table)
 
     def forward(self, h):
-        return ops.linear(h, self.weight, out_dtype=torch.float32)
+        logits = ops.linear(h, self.weight, out_dtype=torch.float32)
+        return logits if self.softcap is None else ops.softcap(logits, self.softcap)

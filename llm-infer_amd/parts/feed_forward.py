@@ -22,7 +22,9 @@ class GatedMLP(Part):
 
     takes_lazy_norm = True      # the normed input goes to ops.linear as it comes
 
-    def __init__(self, *, hidden_size, intermediate_size, activation="silu", prefix, dtype, device):
+    def __init__(self, *, hidden_size, intermediate_size, activation="silu", names=None, prefix, dtype, device):
+        """``names``: local tensor names for gate, up and down."""
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", **(names or {})}
         if activation not in ("silu", "gelu"):
             raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu and gelu are)")
         self.mode = ops.EPI_SWIGLU if activation == "silu" else ops.EPI_GEGLU
@@ -32,16 +34,16 @@ class GatedMLP(Part):
 
     def params(self):
         f, d = self.intermediate_size, self.hidden_size
-        return {"gate_proj.weight": ParamSpec((f, d)), "up_proj.weight": ParamSpec((f, d)),
-                "down_proj.weight": ParamSpec((d, f))}
+        n = self.names
+        return {n["gate"]: ParamSpec((f, d)), n["up"]: ParamSpec((f, d)), n["down"]: ParamSpec((d, f))}
 
     def bind(self, tensors):
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         gu = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
         self.w_gate_up = ops.prepare_weight(gu)
-        self.w_down = ops.prepare_weight(tensors["down_proj.weight"])
+        self.w_down = ops.prepare_weight(tensors[self.names["down"]])
 
     def forward(self, h, residual):
         t = ops.linear(h, self.w_gate_up, self.mode, out_dtype=self.dtype)
@@ -110,7 +112,13 @@ class DenseMLP(Part):
 @register_feed_forward("routed_experts")
 class RoutedExperts(Part):
     """A mixture of ``n_experts`` gated feed-forwards down(silu(gate(h)) * up(h)) of width ``expert_ff`` (tensors
-    ``e<i>.gate``, ``e<i>.up``, ``e<i>.down``), of which every token uses ``top``.
+    ``e<i>.gate``, ``e<i>.up``, ``e<i>.down``), of which every token uses ``top``.  ``gated`` False: an expert is
+    down(act(up(h))) with ``activation`` one of gelu, gelu_tanh, silu, relu2 (the square of relu), and has no gate
+    matrix.  ``scores`` "sigmoid": s is the sigmoid of every router logit instead of their softmax; ``renormalize``
+    False: a chosen expert's weight is its own s (times ``route_scale``), not divided by the sum of the chosen;
+    ``weight_on`` "input": the weight multiplies what the expert reads, the result is the sum of expert(weight * h)
+    (experts without a gate: their up product is linear, so the weight is applied to its sums, act(weight * up(h)),
+    in float32).
 
     The router has n_experts + ``n_identity`` outputs; its logits and everything after them are float32:
     s = softmax(W_router h); the ``top`` outputs with the largest s + correction are chosen (``correction``: a
@@ -135,9 +143,18 @@ class RoutedExperts(Part):
     GROUPED_FROM = 256
 
     def __init__(self, *, hidden_size, n_experts, expert_ff, top, n_identity=0, route_scale=1.0, correction=True,
-                 shared_ff=0, shared_gate=True, names=None, prefix, dtype, device):
+                 shared_ff=0, shared_gate=True, gated=True, activation="silu", scores="softmax", renormalize=True,
+                 weight_on="output", names=None, prefix, dtype, device):
         if not 1 <= top <= n_experts + n_identity:
             raise ValueError(f"routed experts: top {top} of {n_experts + n_identity} outputs")
+        if scores not in ("softmax", "sigmoid") or weight_on not in ("output", "input"):
+            raise ValueError("routed experts: scores 'softmax' or 'sigmoid', weight_on 'output' or 'input'")
+        if gated and (activation != "silu" or weight_on != "output"):
+            raise ValueError("routed experts: gated experts are built with silu and the weight on their output")
+        if not gated and activation not in ops.ACTIVATIONS:
+            raise ValueError(f"routed experts: activation {activation!r} is not built ({', '.join(ops.ACTIVATIONS)} are)")
+        self.gated, self.activation, self.sigmoid_scores = bool(gated), activation, scores == "sigmoid"
+        self.renormalize, self.on_input = bool(renormalize), weight_on == "input"
         self.hidden_size, self.n_experts, self.expert_ff, self.top = hidden_size, n_experts, expert_ff, top
         self.n_identity, self.route_scale, self.correction = n_identity, float(route_scale), bool(correction)
         self.shared_ff, self.shared_gate = int(shared_ff or 0), bool(shared_gate) and bool(shared_ff)
@@ -157,7 +174,9 @@ class RoutedExperts(Part):
         if self.correction:
             out[n["correction"]] = ParamSpec((self.n_experts + self.n_identity,), "vector", "small")
         for p, f in self._experts():
-            out.update({p + n["gate"]: ParamSpec((f, d)), p + n["up"]: ParamSpec((f, d)), p + n["down"]: ParamSpec((d, f))})
+            out.update({p + n["up"]: ParamSpec((f, d)), p + n["down"]: ParamSpec((d, f))})
+            if self.gated:
+                out[p + n["gate"]] = ParamSpec((f, d))
         if self.shared_gate:
             out[n["shared_gate"]] = ParamSpec((1, d), "vector", "wide")
         return out
@@ -166,8 +185,11 @@ class RoutedExperts(Part):
         n, d = self.names, self.hidden_size
         gu, down = [], []
         for p, f in self._experts():
-            g, u = tensors[p + n["gate"]], tensors[p + n["up"]]
-            gu.append(torch.stack([g, u], dim=1).reshape(2 * f, d))            # row 2j: gate_j, row 2j + 1: up_j
+            u = tensors[p + n["up"]]
+            if self.gated:
+                gu.append(torch.stack([tensors[p + n["gate"]], u], dim=1).reshape(2 * f, d))   # row 2j: gate_j, row 2j + 1: up_j
+            else:
+                gu.append(u.as_subclass(torch.Tensor))
             down.append(tensors[p + n["down"]])
         self.w_gate_up = ops.prepare_weight(torch.cat(gu, 0).contiguous())
         self.w_down = ops.prepare_weight(torch.cat(down, 1).contiguous())
@@ -177,8 +199,9 @@ class RoutedExperts(Part):
         if self.dtype != torch.float32:
             parts, at = [], 0
             for (p, f), g_u, d_ in zip(self._experts(), gu, down):
-                parts.append((self._rows(self.w_gate_up, at, 2 * f, g_u), ops.prepare_weight(d_.contiguous())))
-                at += 2 * f
+                rows = 2 * f if self.gated else f
+                parts.append((self._rows(self.w_gate_up, at, rows, g_u), ops.prepare_weight(d_.contiguous())))
+                at += rows
             self.per_expert = parts
         rows = [tensors[n["router"]].float()] + ([tensors[n["shared_gate"]].float().view(1, d)] if self.shared_gate else [])
         self.w_router = torch.cat(rows, 0).contiguous()                       # float32: the logits are summed in float32
@@ -194,7 +217,26 @@ class RoutedExperts(Part):
             return Tensor.wrap(flat, "tiled", (n, k), stacked.owner, stacked)
         return ops.prepare_weight(own.contiguous())
 
+    def _hidden(self, rows, w_up, weights, idx, col, blocks, ff, tail):
+        """The hidden rows of experts without a gate: the activation of the up product's sums, with the routing weight."""
+        z = ops.linear(rows, w_up, out_dtype=torch.float32)
+        return ops.expert_act(z, weights, blocks, ff, tail, self.activation, self.on_input, self.dtype, idx, col)
+
+    def _grouped_plain(self, h, residual, weights):
+        idx, counts = ops.moe_buckets(weights, self.n_experts)
+        for e, n in enumerate(counts):
+            if n:
+                w_up, w_d = self.per_expert[e]
+                t = self._hidden(ops.gather_rows(h, idx[e], n), w_up, weights, idx[e], e, 1, self.expert_ff, 0)
+                ops.scatter_add_rows(residual, ops.linear(t, w_d, out_dtype=torch.float32), idx[e], weights, None)
+        if self.shared_ff:
+            w_up, w_d = self.per_expert[self.n_experts]
+            t = self._hidden(h, w_up, weights, None, self.n_experts, 1, self.shared_ff, 0)
+            ops.linear(t, w_d, ops.EPI_ADD, out=residual)
+
     def _grouped(self, h, residual, weights):
+        if not self.gated:
+            return self._grouped_plain(h, residual, weights)
         idx, counts = ops.moe_buckets(weights, self.n_experts)
         for e, n in enumerate(counts):
             if n:
@@ -209,10 +251,14 @@ class RoutedExperts(Part):
     def forward(self, h, residual):
         logits = ops.small_logits(h, self.w_router)
         weights = ops.moe_route(logits, self.bias, h, residual, self.n_experts + self.n_identity, self.n_experts, self.top,
-                                (1 if self.shared_gate else 2) if self.shared_ff else 0, self.route_scale)
+                                (1 if self.shared_gate else 2) if self.shared_ff else 0, self.route_scale,
+                                self.sigmoid_scores, self.renormalize)
         if (self.per_expert is not None and self.n_experts and h.shape[0] * self.top >= self.GROUPED_FROM * self.n_experts
                 and not torch.cuda.is_current_stream_capturing()):
             return self._grouped(h, residual, weights)
+        if not self.gated:
+            t = self._hidden(h, self.w_gate_up, weights, None, None, self.n_experts, self.expert_ff, self.shared_ff)
+            return ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)
         t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)
         ops.scale_blocks(t, weights, self.n_experts, self.expert_ff, self.shared_ff)
         ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)

@@ -30,7 +30,7 @@ class WeightError(ValueError):
 class ParamSpec:
     shape: tuple
     kind: str = "matrix"        # "matrix" | "vector" | "int"
-    init: str = "normal"        # random-weights mode: "normal" N(0, 0.02) | "ones" 1 + N(0, 0.01) | "small" | "half" | "wide"
+    init: str = "normal"        # random-weights mode: "normal" N(0, 0.02) | "ones" 1 + N(0, 0.01) | "small" | "half" | "wide" | "mean"
 
 
 class Checkpoint:

@@ -2,7 +2,8 @@
 
 Matrices and tables are N(0, 0.02), norm vectors 1 + N(0, 0.01); a vector whose ``init`` is "small" is
 N(0, 0.02) (a bias), one whose ``init`` is "half" 0.5 + N(0, 0.1) within [0, 1] (mixing weights), one whose ``init``
-is "wide" N(0, 0.4) (a short convolution).  Every tensor
+is "wide" N(0, 0.4) (a short convolution), one whose ``init`` is "mean" (1 + N(0, 0.2)) / its length (the weights of
+an average).  Every tensor
 has a generator of its own, seeded by (seed, tensor name), so a tensor's values
 depend on neither the order nor the presence of the others.  The reference has
 no such mode.
@@ -34,6 +35,9 @@ def random_tensor(name: str, spec, seed: int, matrix_dtype: torch.dtype, device=
         return MATRIX_STD * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
     if spec.init == "wide":          # weights of a short convolution and the like: of the order of one half
         return 0.4 * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
+    if spec.init == "mean":          # weights of an average: around 1 / their number
+        n = max(1, spec.shape[0] if spec.shape else 1)
+        return (1.0 + 0.2 * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)) / n
     if spec.init == "half":          # mixing weights between 0 and 1
         return (0.5 + 0.1 * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)).clamp_(0.0, 1.0)
     if spec.kind == "vector" or spec.init == "ones":
