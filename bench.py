@@ -62,7 +62,7 @@ def main() -> int:
                     help="leave out the long contexts, batch 128 and the generation run that the default run adds to points")
     ap.add_argument("--generate", type=int, default=0,
                     help="also generate for this many 128-token prompts with budgets drawn from 16..512 tokens")
-    ap.add_argument("--compare", default="", choices=["", "manirax", "risonex"],
+    ap.add_argument("--compare", default="", choices=["", "manirax", "risonex", "dupolorn"],
                     help="instead of the default workload: prefill and decode throughput of this design at a few "
                          "layer sizes beside the Llama decoder at equal sizes (random weights, a few layers each)")
     ap.add_argument("--sizes", default="", help="with --compare: the layer sizes to run, comma separated (default: all)")
@@ -163,6 +163,24 @@ def compare_configs(design: str, size: dict, layers: int, context: int) -> dict:
         other = {"architecture": "Risonex", "embedding": {"scale": 1.0}, "layers": stack, "norm": {"eps": 1e-5},
                  "vocab": size["vocab"], "width": w, "max_positions": context}
         return {"llama": llama, design: other}
+    if design == "dupolorn":
+        # latent attention of the same heads (hd unrotated and hd / 2 rotated query dimensions a head, values a head wide, a
+        # latent of 3 hd / 2 so that the one key all heads read is 2 hd wide), three layers in four, two of them with sink and
+        # gate; a matrix memory of H / 4 heads (keys 2 hd wide, values 4 hd) in the fourth; a dense gated feed-forward of
+        # the Llama decoder's width in the first layer, then eight experts of a quarter of it, two of them chosen, beside a
+        # shared one
+        lat = {"heads": H, "dim": hd, "rot_dim": hd // 2, "vdim": hd, "kv_rank": 3 * hd // 2, "scale": (3 * hd // 2) ** -0.5,
+               "rot": {"base": 500000.0, "dims": hd // 2}}
+        mem = {"heads": max(1, H // 4), "dim": 2 * hd, "vdim": 4 * hd, "gate_cap": 15.0}
+        kinds = ["latent_attention_2", "latent_attention_2", "latent_attention", "mlstm"]
+        routed = {"kind": "moe", "expert": {"ff": size["ff"] // 4}, "shared": {"ff": size["ff"] // 4},
+                  "router": {"experts": 8, "top": 2}}
+        stack = [{"type": kinds[i % 4], "mixer": mem if kinds[i % 4] == "mlstm" else lat,
+                  "mlp": {"kind": "dense", "ff": size["ff"]} if i == 0 else routed} for i in range(layers)]
+        other = {"architecture": "Dupolorn", "canon": {"taps": 3},
+                 "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 17}, "scale": 1.0}, "layers": stack,
+                 "logit_softcap": 30.0, "norm": {"eps": 1e-5}, "vocab": size["vocab"], "width": w, "max_positions": context}
+        return {"llama": llama, design: other}
     assert design == "manirax"
     # the attention of the same heads beside a linear attention of half as many heads with states of hd x hd
     layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": size["ff"]},
@@ -218,7 +236,8 @@ def compare(args) -> dict:
                     slots = [engine.alloc_slot() for _ in range(batch)]
                     cache.grow(slots, [start] * batch)
                     for g in cache.groups:
-                        g.storage.normal_(0.0, 1.0)
+                        if g.storage.is_floating_point():      # (integer state, a token id say, stays as it is)
+                            g.storage.normal_(0.0, 1.0)
                     sampler = Sampler(temperature=0.0, seed=0)
                     sampler.start(cache, slots, list(range(batch)))
                     runner = engine.decode_runner(sampler, use_graph=True)

@@ -28,7 +28,12 @@ struct MapPages {
     int max_pages;
 };
 
-template <class T, int MAPS, bool PROMPT>
+// HC (decode steps, several query heads on a key/value head): the 32 columns of a tile are 32 query heads of one
+// key/value head for one token instead of 32 tokens of one head, so the keys and values of a token are fetched once for
+// all of them; the four waves of the workgroup share the token's keys and merge all 32 columns' states.
+// One map needs no second half of a weight (nothing is subtracted afterwards): a weight enters the second product
+// rounded once, as in the softmax attention of the other decoders.
+template <class T, int MAPS, bool PROMPT, bool HC>
 __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, const int* __restrict__ tile_t0, const int* __restrict__ tile_n, int H, int G,
@@ -48,9 +53,14 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     // the waves of a workgroup: the query heads of one KV head on the same tile (they fetch the same keys and
     // values, which then come from the CU's cache), or, `split`, shares of the keys of a tile of one token
-    const int h = split ? group : group * nw + wave;
+    const int per_kv = H / G, hc_tiles = (per_kv + 31) / 32;
+    // HC: this lane's head, the column's; h itself may lie beyond the key/value head's last (such a column has no query)
+    const int h = HC ? (group / hc_tiles) * per_kv + (group % hc_tiles) * 32 + col : (split ? group : group * nw + wave);
+    const bool head_ok = !HC || (group % hc_tiles) * 32 + col < per_kv;
+    const int hq = head_ok ? h : (group / hc_tiles) * per_kv;          // a head that exists, for addresses
     const int kwave = split ? wave : 0, kstep = split ? nw : 1;
-    const int g = h / (H / G);
+    const int g = HC ? group / hc_tiles : h / per_kv;
+    constexpr bool SPLIT_W = MAPS == 2;
     // an item of a prompt is two tiles, one that sees many keys and one that sees few (the host pairs them), so that
     // every wave has about the same work; a decode step's item is its one token
     constexpr int parts = PROMPT ? 2 : 1;
@@ -58,7 +68,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const int t0 = PROMPT ? tile_t0[parts * item + part] : item, n = PROMPT ? tile_n[parts * item + part] : 1;
     if (n <= 0) continue;
     const int p0 = pos[t0];                            // the tile's tokens stand at p0, p0 + 1, ...
-    const bool has_query = col < n;
+    const bool has_query = HC ? head_ok : col < n;
     const int pq = p0 + min(col, n - 1);
     int lo_q = block > 0 ? pq - pq % block : 0;
     if (window > 0) lo_q = max(lo_q, pq - window + 1);
@@ -73,7 +83,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
 
     v8 qf[MAPS][D16];
     {
-        const T* qrow = q + ((int64_t)(t0 + min(col, n - 1)) * H + h) * KW;
+        const T* qrow = q + ((int64_t)(t0 + (HC ? 0 : min(col, n - 1))) * H + hq) * KW;
 #pragma unroll
         for (int a = 0; a < MAPS; ++a)
 #pragma unroll
@@ -170,7 +180,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
                 for (int i = 0; i < 8; ++i) {
                     const T hi = from_f32<T>(pr[8 * u + i]);
                     phi[a][u][i] = hi;
-                    plo[a][u][i] = from_f32<T>(pr[8 * u + i] - to_f32(hi));
+                    if (SPLIT_W) plo[a][u][i] = from_f32<T>(pr[8 * u + i] - to_f32(hi));
                 }
         }
 #pragma unroll
@@ -180,17 +190,17 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
 #pragma unroll
                 for (int a = 0; a < MAPS; ++a) {
                     o[a][b] = mfma32(vf[b][u], phi[a][u], o[a][b]);
-                    o[a][b] = mfma32(vf[b][u], plo[a][u], o[a][b]);
+                    if (SPLIT_W) o[a][b] = mfma32(vf[b][u], plo[a][u], o[a][b]);
                 }
             }
     }
     if (split && nw > 1) {
         // a tile of one token whose keys the waves have shared: wave 0 adds up their states in wave order
         constexpr int W = 2 + VALUE_DIM;
-        if (col == 0) {
+        if (HC || col == 0) {
 #pragma unroll
             for (int a = 0; a < MAPS; ++a) {
-                float* mine = lds + (wave * MAPS + a) * W;
+                float* mine = lds + ((wave * MAPS + a) * (HC ? 32 : 1) + (HC ? col : 0)) * W;
                 if (half == 0) { mine[0] = m[a]; mine[1] = l[a]; }
 #pragma unroll
                 for (int b = 0; b < DVB; ++b)
@@ -200,18 +210,19 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
         }
         __syncthreads();
         if (wave != 0) return;
-        if (col == 0) {
+        if (HC || col == 0) {
+            const int cs = HC ? 32 : 1, c0 = HC ? col : 0;
 #pragma unroll
             for (int a = 0; a < MAPS; ++a) {
                 float M = -INFINITY;
-                for (int w = 0; w < nw; ++w) M = fmaxf(M, lds[(w * MAPS + a) * W]);
+                for (int w = 0; w < nw; ++w) M = fmaxf(M, lds[((w * MAPS + a) * cs + c0) * W]);
                 float L = 0.f;
 #pragma unroll
                 for (int b = 0; b < DVB; ++b)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) o[a][b][r] = 0.f;
                 for (int w = 0; w < nw; ++w) {
-                    const float* theirs = lds + (w * MAPS + a) * W;
+                    const float* theirs = lds + ((w * MAPS + a) * cs + c0) * W;
                     if (theirs[0] == -INFINITY) continue;
                     const float f = __builtin_amdgcn_exp2f(theirs[0] - M);
                     L += theirs[1] * f;
@@ -226,7 +237,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     }
     if (sink) {
         // the sink joins every map's sum as one more weight, exp(sink - maximum), with nothing to add to the output
-        const float s2 = sink[h] * 1.4426950408889634f;
+        const float s2 = sink[hq] * 1.4426950408889634f;
 #pragma unroll
         for (int a = 0; a < MAPS; ++a) {
             const float M = fmaxf(m[a], s2), f = __builtin_amdgcn_exp2f(m[a] - M);
@@ -253,7 +264,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     ss += __shfl_xor(ss, 32, WAVE);
     const float rr = out_eps >= 0.f ? out_scale / sqrtf(ss / (float)dv + out_eps) : out_scale;
     if (has_query) {
-        T* orow = out + ((int64_t)(t0 + col) * H + h) * dv;
+        T* orow = out + ((int64_t)(t0 + (HC ? 0 : col)) * H + hq) * dv;
 #pragma unroll
         for (int b = 0; b < DVB; ++b)
 #pragma unroll
@@ -284,12 +295,21 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
     // a workgroup are query heads of one KV head (4, 2 or 1 of them)
     const int split = tile_t0 ? 0 : 1, per_kv = H / G;
     const int heads = split ? 1 : (per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1));
-    dim3 grid(n_tiles, H / heads);
+    // a decode step with four or more query heads on a key/value head: the heads are a tile's columns
+    const bool hc = split && per_kv >= 4;
+    dim3 grid(n_tiles, hc ? G * ((per_kv + 31) / 32) : H / heads);
     const int threads = split ? 256 : 64 * heads;
-    const size_t lds = split ? (size_t)4 * maps * (2 + VALUE_DIM) * sizeof(float) : 0;
-#define GO1(T, M, P) diff_attn_mfma_kernel<T, M, P><<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, \
-                                                                          tile_n, H, G, dv, scale, block, window, lambda, out_eps, out_scale, split, sink)
-#define GO(T, M) do { if (split) GO1(T, M, false); else GO1(T, M, true); } while (0)
+    const size_t lds = split ? (size_t)4 * maps * (hc ? 32 : 1) * (2 + VALUE_DIM) * sizeof(float) : 0;
+#define GO1(T, M, P, C)                                                                                                              \
+    do {                                                                                                                             \
+        auto kfn = diff_attn_mfma_kernel<T, M, P, C>;                                                                                \
+        if (lds > 48 * 1024 &&                                                                                                       \
+            hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)              \
+            return LI_HIP_ERROR;                                                                                                     \
+        kfn<<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, tile_n, H, G, dv, scale, block, window, \
+                                            lambda, out_eps, out_scale, split, sink);                                                \
+    } while (0)
+#define GO(T, M) do { if (hc) GO1(T, M, false, true); else if (split) GO1(T, M, false, false); else GO1(T, M, true, false); } while (0)
     if (dt == DT_F16) { if (maps == 1) GO(f16, 1); else GO(f16, 2); }
     else { if (maps == 1) GO(bf16, 1); else GO(bf16, 2); }
 #undef GO

@@ -201,11 +201,15 @@ extern "C" int li_latent_store(const float* proj, int stride, int q_col, int kv_
 }
 
 // ---------------------------------------------------------------------------
-// A small product per head: out[t][h][j] = sum over i of W[h][i][j] * in[t][h][i]   (W stored [H, n_in, n_out], so that
-// neighbouring threads read neighbouring weights), i < n_in, j < n_out.  Rows of `in` and `out` are addressed by a
+// A small product per head: out[t][h][j] = sum over i of W[h][j][i] * in[t][h][i]   (W stored [H, n_out, n_in]), i < n_in,
+// j < n_out.  Rows of `in` and `out` are addressed by a
 // stride per token and one per head, so that a head's part may lie inside a wider row.  `gate` not null: the result
 // is multiplied by sigmoid(gate[t][h * n_out + j]) (float32 rows, `gate_stride` apart).  Sums are float32.
-// A workgroup takes 16 tokens of one head: their inputs wait in LDS and every thread owns outputs j.
+// head_linear_kernel (float32 models, and whatever the other does not take): a workgroup takes 16 tokens of one head,
+// their inputs wait in LDS and every thread owns outputs j.  head_linear_mfma_kernel (16-bit models): a wave owns 32
+// outputs x 32 tokens of one head, W^T as operand A and the tokens' inputs (rounded to the 16-bit type where they
+// come in float32, as the sum of two such numbers) as operand B of the 32x32x16 matrix instruction, both read straight from memory, 16 bytes a lane
+// where n_in and the rows allow; the four waves of a workgroup take four blocks of outputs for the same tokens.
 // ---------------------------------------------------------------------------
 #define HL_TOK 16
 
@@ -228,7 +232,7 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TI* __restrict__
 #pragma unroll
         for (int k = 0; k < HL_TOK; ++k) acc[k] = 0.f;
         for (int i = 0; i < n_in; ++i) {
-            const float w = to_f32(Wh[(int64_t)i * n_out + j]);
+            const float w = to_f32(Wh[(int64_t)j * n_in + i]);
 #pragma unroll
             for (int k = 0; k < HL_TOK; ++k) acc[k] += w * xs[k * n_in + i];
         }
@@ -243,11 +247,85 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TI* __restrict__
     }
 }
 
+template <class TI, class T>
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(const TI* __restrict__ in, int64_t in_st, int in_sh,
+                                                               const T* __restrict__ W, T* __restrict__ out, int64_t out_st,
+                                                               int out_sh, const float* __restrict__ gate, int64_t gate_st,
+                                                               int n_tokens, int n_in, int n_out, int vec) {
+    typedef typename Vec<T>::v8 v8;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+    const int t = blockIdx.x * 32 + col, h = blockIdx.y, j0 = (blockIdx.z * 4 + wave) * 32;
+    if (j0 >= n_out) return;
+    const bool t_ok = t < n_tokens, j_ok = j0 + col < n_out;
+    const T* wrow = W + ((int64_t)h * n_out + (j_ok ? j0 + col : 0)) * n_in;
+    const TI* xrow = in + (int64_t)(t_ok ? t : 0) * in_st + (int64_t)h * in_sh;
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int k0 = 0; k0 < n_in; k0 += 16) {
+        const int i0 = k0 + 8 * half;
+        v8 a, b, b2;                     // b2: what the rounding of a float32 input leaves, so that the product sees 16 bits of it
+        float xf[8];
+        if (vec && i0 + 8 <= n_in) {
+            a = *(const v8*)(wrow + i0);
+            if (sizeof(TI) == 4) {
+                const f32x4 lo = *(const f32x4*)((const float*)xrow + i0), hi = *(const f32x4*)((const float*)xrow + i0 + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { xf[e] = lo[e]; xf[4 + e] = hi[e]; }
+            } else {
+                b = *(const v8*)((const T*)xrow + i0);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                a[e] = i0 + e < n_in ? wrow[i0 + e] : from_f32<T>(0.f);
+                xf[e] = i0 + e < n_in ? to_f32(xrow[i0 + e]) : 0.f;
+                if (sizeof(TI) != 4) b[e] = from_f32<T>(xf[e]);
+            }
+        }
+        if (sizeof(TI) == 4) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { b[e] = from_f32<T>(xf[e]); b2[e] = from_f32<T>(xf[e] - to_f32(b[e])); }
+        }
+        if (!j_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] = from_f32<T>(0.f);
+        }
+        acc = mfma32(a, b, acc);
+        if (sizeof(TI) == 4) acc = mfma32(a, b2, acc);
+    }
+    if (!t_ok) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int j = j0 + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (j < n_out) {
+            float v = acc[r];
+            if (gate) v *= lt_sigmoid(gate[(int64_t)t * gate_st + (int64_t)h * n_out + j]);
+            out[(int64_t)t * out_st + (int64_t)h * out_sh + j] = from_f32<T>(v);
+        }
+    }
+}
+
 extern "C" int li_head_linear(const void* in, int in_dt, int64_t in_st, int in_sh, const void* W, int w_dt, void* out,
                               int64_t out_st, int out_sh, const float* gate, int64_t gate_st, int n_tokens, int H, int n_in,
                               int n_out, hipStream_t stream) {
     if (n_tokens <= 0) return LI_OK;
     if (H <= 0 || n_in <= 0 || n_out <= 0) return LI_BAD_ARG;
+    if (w_dt == DT_F16 || w_dt == DT_BF16) {
+        // 16 bytes a lane where every fragment begins at a multiple of 16 bytes
+        const int isz = in_dt == DT_F32 ? 4 : 2;
+        const int vec = n_in % 8 == 0 && (uintptr_t)W % 16 == 0 && (uintptr_t)in % 16 == 0 && (in_st * isz) % 16 == 0 &&
+                        ((int64_t)in_sh * isz) % 16 == 0;
+        dim3 grid((n_tokens + 31) / 32, H, (n_out + 127) / 128);
+#define GOM(TI, T) head_linear_mfma_kernel<TI, T><<<grid, 256, 0, stream>>>((const TI*)in, in_st, in_sh, (const T*)W, (T*)out, out_st, \
+                                                                           out_sh, gate, gate_st, n_tokens, n_in, n_out, vec)
+        if (in_dt == DT_F32) { if (w_dt == DT_F16) GOM(float, f16); else GOM(float, bf16); }
+        else if (in_dt == w_dt) { if (w_dt == DT_F16) GOM(f16, f16); else GOM(bf16, bf16); }
+        else return LI_BAD_ARG;
+#undef GOM
+        LI_CHECK_LAUNCH();
+        return LI_OK;
+    }
     const size_t lds = (size_t)HL_TOK * n_in * sizeof(float);
     if (lds > 64000) return LI_UNSUPPORTED;
     dim3 grid((n_tokens + HL_TOK - 1) / HL_TOK, H);
@@ -266,109 +344,229 @@ extern "C" int li_head_linear(const void* in, int in_dt, int64_t in_st, int in_s
 // The matrix memory (mLSTM) recurrence.  Per sequence and head, with q_t, k_t [d] and v_t [dv] from the float32 rows
 // `proj` (q is multiplied by qscale), the raw gates gi, gf from two more columns, cap > 0:
 //   i = cap tanh((gi + bi[h]) / cap),   f = logsigmoid(cap tanh((gf + bf[h]) / cap))
-//   m_t = max(f + m_{t-1}, i);   a = exp(f + m_{t-1} - m_t),  b = exp(i - m_t)
-//   S_t = a S_{t-1} + b k_t v_t^T;   n_t = a n_{t-1} + b k_t;   y_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
+//   m_t = max(f + m_{t-1}, i);   a_t = exp(f + m_{t-1} - m_t),  b_t = exp(i - m_t)
+//   S_t = a_t S_{t-1} + b_t k_t v_t^T;   n_t = a_t n_{t-1} + b_t k_t;   y_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
 // S [d, dv], n [d] and m are float32 state of every sequence (`S_state` [slots, H, d, dv]; `nm_state` [slots, H, d + 1]
-// with m behind n), zero when it starts (so m_0 = 0).  One wave per (sequence, head, 64 columns of dv): a lane keeps
-// its column of S in registers for all the tokens that the sequence brings; q_t, k_t and n lie across the lanes and
-// reach every lane by lane reads.  The waves of a head all begin from the n and m that the step found, so the new
-// ones go to scratch memory `nm_new` [sequences, H, d + 1] first and mlstm_commit_kernel puts them into the state once
-// every wave has ended.  y float32 [T, H * dv].
+// with m behind n), zero when it starts (so m_0 = 0).
+// Two kernels come first.  mlstm_gates_kernel, a thread per (token, head): i and f into `coef` [T, H, 3].
+// mlstm_max_kernel, a wave per (sequence, head), walks the sequence's tokens with the one dependent chain there is,
+// m_t, and leaves (a_t, b_t, exp(-m_t)) in `coef` and the last m in the state.  With a_t and b_t known the
+// recurrence of S and n is linear, with one decay for all of a head's elements.
+// mlstm_scan_kernel, one wave per (sequence or segment, head, 64 columns of dv): a lane keeps its column of S in
+// registers for all the tokens of its stretch; q_t, k_t and n lie across the lanes and reach every lane by lane reads.
+// PASS 0 walks a sequence's tokens in order from the state and leaves the state up to date (the waves of a head all
+// begin from the n that the step found, so the new one goes to `nm_new` [sequences, H, d + 1] first and
+// mlstm_commit_kernel puts it into the state once every wave has ended).  A prompt may also be walked in segments
+// side by side (ScanSegments): PASS 1 runs every segment from zero and leaves what it adds to S and n and the product
+// of its a_t; seg_combine_kernel walks a sequence's segments in order, X <- A_seg X + D_seg, leaving the value
+// before every segment where its contribution was; PASS 3 runs every segment again from there and writes y.
+// y float32 [T, H * dv].
 // ---------------------------------------------------------------------------
-template <int NMAX>
-__global__ __launch_bounds__(64) void mlstm_scan_kernel(
-    const float* __restrict__ proj, int stride, int q_col, int k_col, int v_col, int i_col, int f_col,
-    const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float qscale,
-    float* __restrict__ S_state, const float* __restrict__ nm_state, float* __restrict__ nm_new,
-    const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart, const int* __restrict__ seq_qlen, float* __restrict__ y, int H, int d, int dv) {
-    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, col = blockIdx.z * 64 + lane;
+__global__ void mlstm_gates_kernel(const float* __restrict__ proj, int stride, int i_col, int f_col,
+                                   const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
+                                   float* __restrict__ coef, int n_tokens, int H) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_tokens * H) return;
+    const int t = e / H, h = e - t * H;
+    const float gi = proj[(int64_t)t * stride + i_col + h] + (i_bias ? i_bias[h] : 0.f);
+    const float gf = proj[(int64_t)t * stride + f_col + h] + (f_bias ? f_bias[h] : 0.f);
+    coef[(int64_t)e * 3] = cap * tanhf(gi / cap);
+    coef[(int64_t)e * 3 + 1] = lt_logsigmoid(cap * tanhf(gf / cap));
+}
+
+__global__ __launch_bounds__(64) void mlstm_max_kernel(float* __restrict__ coef, float* __restrict__ nm_state,
+                                                       const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
+                                                       const int* __restrict__ seq_qlen, int H, int d) {
+    // one wave per (sequence, head), 64 tokens at a time: every lane fetches its token's i and f, the chain runs over
+    // lane reads (no memory in it), each lane keeps the maximum before and after its own token and finishes it alone
+    const int seq = blockIdx.x / H, h = blockIdx.x - seq * H, lane = threadIdx.x;
     const int q0 = seq_qstart ? seq_qstart[seq] : seq, n = seq_qlen ? seq_qlen[seq] : 1;
-    const int slot = seq_slot[seq];
+    if (n <= 0) return;
+    float* mp = nm_state + ((int64_t)seq_slot[seq] * H + h) * (d + 1) + d;
+    float m = *mp;
+    for (int base = 0; base < n; base += 64) {
+        const int t = base + lane, cnt = min(64, n - base);
+        float* c = coef + ((int64_t)(q0 + min(t, n - 1)) * H + h) * 3;
+        const float ig = c[0], fg = c[1];
+        float before = 0.f, after = 0.f;
+        for (int j = 0; j < cnt; ++j) {
+            const float fj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fg), j));
+            const float ij = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ig), j));
+            const float mn = fmaxf(fj + m, ij);
+            if (lane == j) { before = m; after = mn; }
+            m = mn;
+        }
+        if (t < n) {
+            c[0] = expf(fg + before - after);
+            c[1] = expf(ig - after);
+            c[2] = expf(-after);
+        }
+    }
+    if (lane == 0) *mp = m;
+}
+
+struct ScanSegments {
+    const int* seg_seq;         // [segments] the sequence of a segment
+    const int* seg_t0;          // [segments] its first token among the sequence's tokens of this step
+    const int* seg_n;           // [segments] its tokens
+    float* seg_S;               // [segments, H, d, dv]
+    float* seg_nrm;             // [segments, H, d]
+    float* seg_decay;           // [segments, H]
+};
+
+template <int NMAX, int PASS>
+__global__ __launch_bounds__(64) void mlstm_scan_kernel(
+    const float* __restrict__ proj, int stride, int q_col, int k_col, int v_col, const float* __restrict__ coef,
+    float qscale, float* __restrict__ S_state, const float* __restrict__ nm_state, float* __restrict__ nm_new,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart, const int* __restrict__ seq_qlen,
+    float* __restrict__ y, int H, int d, int dv, ScanSegments sg) {
+    const int h = blockIdx.y, lane = threadIdx.x, col = blockIdx.z * 64 + lane;
     const bool live = col < dv;
-    float* S = S_state + (((int64_t)slot * H + h) * d) * dv + col;
-    const float* nm = nm_state + ((int64_t)slot * H + h) * (d + 1);
+    int q0, n;
+    float* S;
+    const float* nsrc;
+    if (PASS == 0) {
+        const int seq = blockIdx.x;
+        q0 = seq_qstart ? seq_qstart[seq] : seq;
+        n = seq_qlen ? seq_qlen[seq] : 1;
+        S = S_state + (((int64_t)seq_slot[seq] * H + h) * d) * dv + col;
+        nsrc = nm_state + ((int64_t)seq_slot[seq] * H + h) * (d + 1);
+    } else {
+        const int seg = blockIdx.x;
+        q0 = seq_qstart[sg.seg_seq[seg]] + sg.seg_t0[seg];
+        n = sg.seg_n[seg];
+        S = sg.seg_S + (((int64_t)seg * H + h) * d) * dv + col;
+        nsrc = sg.seg_nrm + ((int64_t)seg * H + h) * d;
+    }
+    if (n <= 0) return;
     constexpr int NV = (NMAX + 63) / 64;
     float s[NMAX], nl[NV];
 #pragma unroll
-    for (int i = 0; i < NMAX; ++i) s[i] = (live && i < d) ? S[(int64_t)i * dv] : 0.f;
+    for (int i = 0; i < NMAX; ++i) s[i] = (PASS != 1 && live && i < d) ? S[(int64_t)i * dv] : 0.f;
 #pragma unroll
-    for (int v = 0; v < NV; ++v) nl[v] = v * 64 + lane < d ? nm[v * 64 + lane] : 0.f;
-    float m = nm[d];
-    const float bi = i_bias ? i_bias[h] : 0.f, bf = f_bias ? f_bias[h] : 0.f;
-    float qv[NV], kv[NV], x = 0.f, gi = 0.f, gf = 0.f;
+    for (int v = 0; v < NV; ++v) nl[v] = (PASS != 1 && v * 64 + lane < d) ? nsrc[v * 64 + lane] : 0.f;
+    float qv[NV], kv[NV], x = 0.f, ca = 0.f, cb = 0.f, cm = 0.f, decay = 1.f;
     auto fetch = [&](int t) {
         const float* __restrict__ row = proj + (int64_t)(q0 + t) * stride;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int i = v * 64 + lane;
-            qv[v] = i < d ? row[q_col + h * d + i] * qscale : 0.f;
+            if (PASS != 1) qv[v] = i < d ? row[q_col + h * d + i] * qscale : 0.f;
             kv[v] = i < d ? row[k_col + h * d + i] : 0.f;
         }
         x = live ? row[v_col + h * dv + col] : 0.f;
-        gi = row[i_col + h];
-        gf = row[f_col + h];
+        const float* c = coef + ((int64_t)(q0 + t) * H + h) * 3;
+        ca = c[0]; cb = c[1]; cm = c[2];
     };
-    if (n > 0) fetch(0);
+    fetch(0);
     for (int t = 0; t < n; ++t) {
         float qt[NV], kt[NV];
 #pragma unroll
-        for (int v = 0; v < NV; ++v) { qt[v] = qv[v]; kt[v] = kv[v]; }
-        const float xt = x;
-        const float ig = cap * tanhf((gi + bi) / cap), fg = lt_logsigmoid(cap * tanhf((gf + bf) / cap));
+        for (int v = 0; v < NV; ++v) { qt[v] = PASS != 1 ? qv[v] : 0.f; kt[v] = kv[v]; }
+        const float a = ca, b = cb, em = cm, bx = cb * x;
         if (t + 1 < n) fetch(t + 1);
-        const float mn = fmaxf(fg + m, ig);
-        const float a = expf(fg + m - mn), b = expf(ig - mn);
-        m = mn;
+        decay *= a;
         float nq = 0.f;
 #pragma unroll
         for (int v = 0; v < NV; ++v) { nl[v] = a * nl[v] + b * kt[v]; nq += nl[v] * qt[v]; }
-        nq = wave_sum(nq);
-        const float bx = b * xt;
+        if (PASS != 1) nq = wave_sum(nq);
         float acc = 0.f;
 #pragma unroll
         for (int i = 0; i < NMAX; ++i) {
             const float kk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(kt[i >> 6]), i & 63));
-            const float qq = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qt[i >> 6]), i & 63));
             s[i] = a * s[i] + kk * bx;
-            acc += s[i] * qq;
+            if (PASS != 1) {
+                const float qq = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qt[i >> 6]), i & 63));
+                acc += s[i] * qq;
+            }
         }
-        if (live) y[(int64_t)(q0 + t) * H * dv + h * dv + col] = acc / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
+        if (PASS != 1 && live) y[(int64_t)(q0 + t) * H * dv + h * dv + col] = acc / (fmaxf(fabsf(nq), em) + 1e-6f);
     }
-    if (n <= 0) return;
+    if (PASS == 3) return;
     if (live) {
 #pragma unroll
         for (int i = 0; i < NMAX; ++i) if (i < d) S[(int64_t)i * dv] = s[i];
     }
     if (blockIdx.z == 0) {
-        float* to = nm_new + ((int64_t)seq * H + h) * (d + 1);
+        float* to = PASS == 0 ? nm_new + ((int64_t)blockIdx.x * H + h) * (d + 1) : sg.seg_nrm + ((int64_t)blockIdx.x * H + h) * d;
 #pragma unroll
         for (int v = 0; v < NV; ++v) if (v * 64 + lane < d) to[v * 64 + lane] = nl[v];
-        if (lane == 0) to[d] = m;
+        if (PASS == 1 && lane == 0) sg.seg_decay[(int64_t)blockIdx.x * H + h] = decay;
     }
 }
 
+// n of every (sequence, head) from the scratch memory into the state (m, behind it, is mlstm_max_kernel's).
 __global__ void mlstm_commit_kernel(const float* __restrict__ nm_new, float* __restrict__ nm_state,
                                     const int* __restrict__ seq_slot, const int* __restrict__ seq_qlen, int H, int d) {
     const int seq = blockIdx.x, h = blockIdx.y;
     if (seq_qlen && seq_qlen[seq] <= 0) return;
     const float* from = nm_new + ((int64_t)seq * H + h) * (d + 1);
     float* to = nm_state + ((int64_t)seq_slot[seq] * H + h) * (d + 1);
-    for (int i = threadIdx.x; i <= d; i += blockDim.x) to[i] = from[i];
+    for (int i = threadIdx.x; i < d; i += blockDim.x) to[i] = from[i];
 }
 
+// One thread per element of a head's state (`per_head` of them, `state_stride` floats from head to head in the
+// state): walks the sequence's segments in order.
+__global__ void seg_combine_kernel(float* __restrict__ state, int64_t state_stride, const int* __restrict__ seq_slot,
+                                   const int* __restrict__ seq_seg0, const int* __restrict__ seq_nseg,
+                                   float* __restrict__ seg_buf, const float* __restrict__ seg_decay, int H, int64_t per_head) {
+    const int seq = blockIdx.x, h = blockIdx.y;
+    const int c0 = seq_seg0[seq], nc = seq_nseg[seq];
+    for (int64_t e = (int64_t)blockIdx.z * blockDim.x + threadIdx.x; e < per_head; e += (int64_t)gridDim.z * blockDim.x) {
+        float* X = state + ((int64_t)seq_slot[seq] * H + h) * state_stride + e;
+        float x = *X;
+        for (int c = c0; c < c0 + nc; ++c) {
+            float* L = seg_buf + ((int64_t)c * H + h) * per_head + e;
+            const float own = *L;
+            *L = x;
+            x = seg_decay[(int64_t)c * H + h] * x + own;
+        }
+        *X = x;
+    }
+}
+
+#define MLSTM_GO(NM, PASS, GRID) mlstm_scan_kernel<NM, PASS><<<GRID, 64, 0, stream>>>(proj, stride, q_col, k_col, v_col, coef, qscale, \
+        S_state, nm_state, nm_new, seq_slot, seq_qstart, seq_qlen, y, H, d, dv, sg)
+#define MLSTM_LAUNCH(PASS, GRID)                                                                             \
+    do {                                                                                                     \
+        if (d <= 16) MLSTM_GO(16, PASS, GRID); else if (d <= 32) MLSTM_GO(32, PASS, GRID);                   \
+        else if (d <= 64) MLSTM_GO(64, PASS, GRID); else if (d <= 128) MLSTM_GO(128, PASS, GRID);            \
+        else MLSTM_GO(256, PASS, GRID);                                                                      \
+    } while (0)
+
+// coef: scratch float32 [T, H, 3]; nm_new: scratch float32 [sequences, H, d + 1].  n_segs > 0 (with the segment lists and
+// scratch seg_S [segments, H, d, dv], seg_nrm [segments, H, d], seg_decay [segments, H]): the tokens run in segments.
 extern "C" int li_mlstm_scan(const float* proj, int stride, int q_col, int k_col, int v_col, int i_col, int f_col,
                              const float* i_bias, const float* f_bias, float cap, float qscale, float* S_state,
-                             float* nm_state, float* nm_new, const int* seq_slot, const int* seq_qstart, const int* seq_qlen, float* y,
-                             int n_seqs, int H, int d, int dv, hipStream_t stream) {
-    if (n_seqs <= 0) return LI_OK;
-    if (H <= 0 || d <= 0 || dv <= 0 || !(cap > 0.f)) return LI_BAD_ARG;
+                             float* nm_state, float* nm_new, float* coef, const int* seq_slot, const int* seq_qstart,
+                             const int* seq_qlen, float* y, int n_tokens, int n_seqs, int H, int d, int dv,
+                             const int* seg_seq, const int* seg_t0, const int* seg_n, const int* seq_seg0,
+                             const int* seq_nseg, int n_segs, float* seg_S, float* seg_nrm, float* seg_decay,
+                             hipStream_t stream) {
+    if (n_seqs <= 0 || n_tokens <= 0) return LI_OK;
+    if (H <= 0 || d <= 0 || dv <= 0 || !(cap > 0.f) || !coef) return LI_BAD_ARG;
     if (d > 256) return LI_UNSUPPORTED;
-    dim3 grid(n_seqs, H, (dv + 63) / 64);
-#define GO(NM) mlstm_scan_kernel<NM><<<grid, 64, 0, stream>>>(proj, stride, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, \
-                                                              qscale, S_state, nm_state, nm_new, seq_slot, seq_qstart, seq_qlen, y, H, d, dv)
-    if (d <= 16) GO(16); else if (d <= 32) GO(32); else if (d <= 64) GO(64); else if (d <= 128) GO(128); else GO(256);
-#undef GO
-    mlstm_commit_kernel<<<dim3(n_seqs, H), 64, 0, stream>>>(nm_new, nm_state, seq_slot, seq_qlen, H, d);
+    mlstm_gates_kernel<<<(n_tokens * H + 255) / 256, 256, 0, stream>>>(proj, stride, i_col, f_col, i_bias, f_bias, cap, coef,
+                                                                       n_tokens, H);
+    mlstm_max_kernel<<<n_seqs * H, 64, 0, stream>>>(coef, nm_state, seq_slot, seq_qstart, seq_qlen, H, d);
+    ScanSegments sg{seg_seq, seg_t0, seg_n, seg_S, seg_nrm, seg_decay};
+    if (n_segs <= 0) {
+        if (!nm_new) return LI_BAD_ARG;
+        dim3 grid(n_seqs, H, (dv + 63) / 64);
+        MLSTM_LAUNCH(0, grid);
+        mlstm_commit_kernel<<<dim3(n_seqs, H), 64, 0, stream>>>(nm_new, nm_state, seq_slot, seq_qlen, H, d);
+    } else {
+        if (!seq_qstart || !seq_qlen || !seg_seq || !seg_t0 || !seg_n || !seq_seg0 || !seq_nseg || !seg_S || !seg_nrm || !seg_decay)
+            return LI_BAD_ARG;
+        dim3 grid(n_segs, H, (dv + 63) / 64);
+        MLSTM_LAUNCH(1, grid);
+        const int64_t per_head = (int64_t)d * dv;
+        seg_combine_kernel<<<dim3(n_seqs, H, (unsigned)((per_head + 255) / 256)), 256, 0, stream>>>(
+            S_state, per_head, seq_slot, seq_seg0, seq_nseg, seg_S, seg_decay, H, per_head);
+        seg_combine_kernel<<<dim3(n_seqs, H, 1), 256, 0, stream>>>(nm_state, d + 1, seq_slot, seq_seg0, seq_nseg, seg_nrm,
+                                                                    seg_decay, H, d);
+        MLSTM_LAUNCH(3, grid);
+    }
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

@@ -1592,16 +1592,17 @@ def latent_store(proj, q_col, kv_col, norm_weight, eps, inv_freq, rot, pos, tok_
 
 
 def head_linear(x, x_col, x_head_stride, w, out, out_col, out_head_stride, gate=None, gate_col=0) -> torch.Tensor:
-    """A product per head: out[t, out_col + h * out_head_stride + j] = sum over i of w[h, i, j] * x[t, x_col + h *
-    x_head_stride + i], ``w`` [H, n_in, n_out] in the model's type, ``x`` [T, ...] float32 or of that type, ``out``
+    """A product per head: out[t, out_col + h * out_head_stride + j] = sum over i of w[h, j, i] * x[t, x_col + h *
+    x_head_stride + i], ``w`` [H, n_out, n_in] in the model's type (a 16-bit model runs it on the matrix cores, a float32
+    input as the sum of two 16-bit numbers), ``x`` [T, ...] float32 or of that type, ``out``
     [T, ...] of that type (both may be wider rows in which a head's part lies).  ``gate`` (float32 rows): the result
     is multiplied by sigmoid(gate[t, gate_col + h * n_out + j]).  Sums are float32."""
     _dev(x, w, out, gate)
     x2, o2 = x.view(x.shape[0], -1), out.view(out.shape[0], -1)
     t = x2.shape[0]
     _need(w.dim() == 3 and w.dtype in DT and x2.dtype in (torch.float32, w.dtype) and o2.dtype == w.dtype and o2.shape[0] == t,
-          "head_linear: weights [H, n_in, n_out], rows of their type (or float32 in)")
-    H, n_in, n_out = w.shape
+          "head_linear: weights [H, n_out, n_in], rows of their type (or float32 in)")
+    H, n_out, n_in = w.shape
     _need(x_col >= 0 and x_col + (H - 1) * x_head_stride + n_in <= x2.shape[1], "head_linear: input columns beyond the rows")
     _need(out_col >= 0 and out_col + (H - 1) * out_head_stride + n_out <= o2.shape[1], "head_linear: output columns beyond the rows")
     if gate is not None:
@@ -1617,12 +1618,15 @@ def head_linear(x, x_col, x_head_stride, w, out, out_col, out_head_stride, gate=
     return out
 
 
-def mlstm_scan(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, q_scale, state, norm_state, ctx, heads, d, dv) -> torch.Tensor:
+def mlstm_scan(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, q_scale, state, norm_state, ctx, heads, d, dv,
+               segments=None) -> torch.Tensor:
     """The matrix-memory recurrence in float32 over the tokens of a step.  q, k [heads, d], v [heads, dv] and the two raw
     gates [heads] are columns of the float32 rows ``proj``; with i = cap tanh((gi + i_bias) / cap), f = logsigmoid(cap
     tanh((gf + f_bias) / cap)):  m <- max(f + m, i);  S <- exp(f + m_old - m) S + exp(i - m) k v^T, n likewise with k;
     y = S^T q / (max(|n . q|, exp(-m)) + 1e-6), q times ``q_scale``.  ``state`` float32 [slots, heads, d, dv] and
-    ``norm_state`` float32 [slots, heads, d + 1] (n, then m) are read and left up to date.  Returns y float32 [T, heads * dv]."""
+    ``norm_state`` float32 [slots, heads, d + 1] (n, then m) are read and left up to date.  ``segments``
+    (``ssm_segments``): the tokens run in segments side by side, each twice (first for what it adds to the state, then,
+    from the state before it, for y); None: every sequence token by token in order.  Returns y float32 [T, heads * dv]."""
     _dev(proj, i_bias, f_bias, state, norm_state)
     _f32_rows(proj, "mlstm projections")
     t = proj.shape[0]
@@ -1635,11 +1639,26 @@ def mlstm_scan(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, q_s
     _need(norm_state.dtype == torch.float32 and tuple(norm_state.shape[1:]) == (heads, d + 1) and norm_state.shape[0] == state.shape[0],
           "mlstm normaliser state: float32 [slots, heads, d + 1]")
     seq_slot, qstart, qlen = _seq_arrays(ctx, t)
-    y = torch.empty((t, heads * dv), dtype=torch.float32, device=proj.device)
-    fresh = torch.empty((ctx.n_seqs, heads, d + 1), dtype=torch.float32, device=proj.device)
+    dev = proj.device
+    y = torch.empty((t, heads * dv), dtype=torch.float32, device=dev)
+    coef = torch.empty((t, heads, 3), dtype=torch.float32, device=dev)
+    fresh = seg = None
+    if segments is None:
+        fresh = torch.empty((ctx.n_seqs, heads, d + 1), dtype=torch.float32, device=dev)
+        tail = (None, None, None, None, None, 0, None, None, None)
+    else:
+        _need(qstart is not None, "mlstm in segments: per-sequence starts and lengths")
+        k = segments["n"]
+        for name, n in (("seg_seq", k), ("seg_t0", k), ("seg_n", k), ("seq_seg0", ctx.n_seqs), ("seq_nseg", ctx.n_seqs)):
+            _i32(segments[name], n, "mlstm " + name)
+        seg = (torch.empty((k, heads, d, dv), dtype=torch.float32, device=dev), torch.empty((k, heads, d), dtype=torch.float32, device=dev),
+               torch.empty((k, heads), dtype=torch.float32, device=dev))
+        tail = (_ptr(segments["seg_seq"]), _ptr(segments["seg_t0"]), _ptr(segments["seg_n"]), _ptr(segments["seq_seg0"]),
+                _ptr(segments["seq_nseg"]), k, _ptr(seg[0]), _ptr(seg[1]), _ptr(seg[2]))
     _check(hybrid().li_mlstm_scan(_ptr(proj), proj.shape[1], q_col, k_col, v_col, i_col, f_col, _ptr(i_bias), _ptr(f_bias),
-                                  c_float(cap), c_float(q_scale), _ptr(state), _ptr(norm_state), _ptr(fresh), _ptr(seq_slot),
-                                  _ptr(qstart), _ptr(qlen), _ptr(y), ctx.n_seqs, heads, d, dv, _stream()), "mlstm_scan")
+                                  c_float(cap), c_float(q_scale), _ptr(state), _ptr(norm_state), _ptr(fresh), _ptr(coef),
+                                  _ptr(seq_slot), _ptr(qstart), _ptr(qlen), _ptr(y), t, ctx.n_seqs, heads, d, dv, *tail, _stream()),
+           "mlstm_scan")
     return y
 
 

@@ -74,10 +74,10 @@ class LatentAttention(Part):
         rows = [tensors[n["q"]], tensors[n["dkv"]]] + ([tensors[n["g"]]] if self.gate else [])
         self.w_in = ops.prepare_weight(torch.cat(rows, 0).contiguous())
         self.wo = ops.prepare_weight(tensors[n["o"]])
-        # the products per head keep their matrices [H, inputs, outputs]: W_uk as stored (a head's d rows of r), W_uv turned
+        # the products per head keep their matrices [H, outputs, inputs]: W_uk turned (a head's d rows of r are its inputs), W_uv as stored
         # (in the model's type also where the file stores them wider: their products run beside 16-bit queries and sums)
-        self.w_uk = tensors[n["uk"]].as_subclass(torch.Tensor).view(H, d, r).to(self.dtype).contiguous() if d else None
-        self.w_uv = tensors[n["uv"]].as_subclass(torch.Tensor).view(H, dv, r).transpose(1, 2).to(self.dtype).contiguous()
+        self.w_uk = tensors[n["uk"]].as_subclass(torch.Tensor).view(H, d, r).transpose(1, 2).to(self.dtype).contiguous() if d else None
+        self.w_uv = tensors[n["uv"]].as_subclass(torch.Tensor).view(H, dv, r).to(self.dtype).contiguous()
         self.kv_norm = tensors[n["kv_norm"]]
         self.sinks = tensors[n["sink"]] if self.sink else None
 

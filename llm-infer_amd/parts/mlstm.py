@@ -25,7 +25,9 @@ class MatrixLSTM(Part):
     Every head's y is divided by its root mean square (``norm_eps``); the heads side by side are multiplied by a
     weight [H dv] and by sigmoid(W_g h), and projected.  S [H, d, dv], n and m are float32 state of every sequence
     (two ``StateSpec``s: S, and n with m behind it), carried from step to step; gates, decays and the recurrence are
-    float32 whatever the matrices' type.  The six input projections are one product against [Wq; Wk; Wv; Wg; Wi; Wf].
+    float32 whatever the matrices' type.  With the maxima m_t known (one short chain per head) the recurrence of S and n is
+    linear, and a 16-bit model walks a long prompt in segments side by side (each twice: for what it adds to the state, then
+    from the state before it).  The six input projections are one product against [Wq; Wk; Wv; Wg; Wi; Wf].
     ``names``: local tensor names."""
 
     takes_lazy_norm = True
@@ -67,7 +69,15 @@ class MatrixLSTM(Part):
         k_col, v_col = H * d, 2 * H * d
         g_col = v_col + H * dv
         i_col = g_col + H * dv
+        # a 16-bit model walks long prompts in segments side by side; a float32 model (and every decode step) walks each
+        # sequence in order, which gives the same bits however a prompt is cut
+        segments = None
+        if self.dtype != torch.float32 and not ctx.is_decode and getattr(ctx, "host_qlens", None):
+            waves_a_token = H * ((dv + 63) // 64)
+            length = max(16, min(ops.SSM_SEGMENT, 1 << max(0, (ctx.n_tokens * waves_a_token // ops.SSM_WAVES).bit_length() - 1)))
+            if max(ctx.host_qlens) > length:
+                segments = ops.ssm_segments(ctx, length)
         y = ops.mlstm_scan(proj, 0, k_col, v_col, i_col, i_col + H, self.i_bias, self.f_bias, self.gate_cap, float(d) ** -0.5,
-                           views[0].state, views[1].state, ctx, H, d, dv)
+                           views[0].state, views[1].state, ctx, H, d, dv, segments)
         a = ops.gated_head_norm(y, self.norm, proj, g_col, H, self.norm_eps, self.dtype)
         ops.linear(a, self.wo, ops.EPI_ADD, out=residual)

@@ -217,14 +217,15 @@ def test_convolution_ahead_of_a_mixer(lib, taps):
 def test_product_per_head_and_gate(lib, dtype):
     from llm_infer_amd.kernels import ops
     g = torch.Generator().manual_seed(3)
-    for T, H, n_in, n_out in ((1, 3, 20, 40), (37, 2, 130, 7), (16, 5, 64, 64)):
-        w = (torch.randn(H, n_in, n_out, generator=g) * n_in ** -0.5).to(DT[dtype])
-        x = torch.randn(T, 11 + H * (n_in + 5), generator=g)
+    for T, H, n_in, n_out in ((1, 3, 20, 40), (37, 2, 130, 7), (16, 5, 64, 64), (70, 3, 192, 200)):
+        w = (torch.randn(H, n_out, n_in, generator=g) * n_in ** -0.5).to(DT[dtype])
+        c0, hs = (16, n_in + 8) if n_in % 8 == 0 else (11, n_in + 5)         # heads at multiples of 16 bytes, and not
+        x = torch.randn(T, c0 + H * hs, generator=g)
         gate = torch.randn(T, 9 + H * n_out, generator=g)
         out = torch.zeros(T, H, n_out + 3, dtype=DT[dtype], device=DEV)
-        ops.head_linear(x.to(DEV), 11, n_in + 5, w.to(DEV), out, 3, n_out + 3, gate=gate.to(DEV), gate_col=9)
-        xin = torch.stack([x[:, 11 + h * (n_in + 5):11 + h * (n_in + 5) + n_in] for h in range(H)], 1).double()
-        ref = torch.einsum("thi,hij->thj", xin, w.double()) * torch.sigmoid(gate[:, 9:].double().view(T, H, n_out))
+        ops.head_linear(x.to(DEV), c0, hs, w.to(DEV), out, 3, n_out + 3, gate=gate.to(DEV), gate_col=9)
+        xin = torch.stack([x[:, c0 + h * hs:c0 + h * hs + n_in] for h in range(H)], 1).double()
+        ref = torch.einsum("thi,hji->thj", xin, w.double()) * torch.sigmoid(gate[:, 9:].double().view(T, H, n_out))
         assert error(out[:, :, 3:].cpu(), ref) < (1e-5 if dtype == "float32" else 3e-2)      # the output is rounded to 16 bits
         assert out[:, :, :3].abs().max() == 0                                 # nothing beside a head's own columns
 
@@ -391,7 +392,7 @@ def test_matrix_memory_carries_a_first_token_far(lib):
     cache = None
     for schedule in ([{"a": n}], [{"a": 2}, {"a": 300}, {"a": 298}], [{"a": 500}] + [{"a": 1}] * 100):
         got, cache = run_mixer(part, {"a": h}, schedule, "float32", cache=cache)
-        assert error(got["a"], ref) < 1e-4, len(schedule)
+        assert error(got["a"], ref) < 3e-4, len(schedule)            # 600 steps of float32 rounding
     assert only.abs().max() > 0
 
 
