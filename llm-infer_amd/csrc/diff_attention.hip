@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, const int* __restrict__ tile_t0, const int* __restrict__ tile_n, int H, int G,
     int dv, float scale, int block, int window, float lambda, float out_eps, float out_scale, int split,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, float* __restrict__ shares_out) {
     typedef typename Vec<T>::v8 v8;
     constexpr int D16 = MAP_DIM / 16, KW = MAPS * MAP_DIM, DVB = VALUE_DIM / 32;
     extern __shared__ float lds[];
@@ -58,7 +58,8 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const int h = HC ? (group / hc_tiles) * per_kv + (group % hc_tiles) * 32 + col : (split ? group : group * nw + wave);
     const bool head_ok = !HC || (group % hc_tiles) * 32 + col < per_kv;
     const int hq = head_ok ? h : (group / hc_tiles) * per_kv;          // a head that exists, for addresses
-    const int kwave = split ? wave : 0, kstep = split ? nw : 1;
+    // HC: the workgroups along the grid's third dimension share a token's keys as the waves of one do
+    const int kwave = split ? (HC ? blockIdx.z * nw + wave : wave) : 0, kstep = split ? (HC ? nw * gridDim.z : nw) : 1;
     const int g = HC ? group / hc_tiles : h / per_kv;
     constexpr bool SPLIT_W = MAPS == 2;
     // an item of a prompt is two tiles, one that sees many keys and one that sees few (the host pairs them), so that
@@ -235,6 +236,23 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
             }
         }
     }
+    if (HC && gridDim.z > 1) {
+        // the keys were shared among workgroups: this one's state goes to `shares_out` [token, head, share, map, 2 + VALUE_DIM]
+        // and diff_attn_merge_kernel finishes
+        constexpr int W = 2 + VALUE_DIM;
+        if (has_query) {
+#pragma unroll
+            for (int a = 0; a < MAPS; ++a) {
+                float* mine = shares_out + ((((int64_t)t0 * H + hq) * gridDim.z + blockIdx.z) * MAPS + a) * W;
+                if (half == 0) { mine[0] = m[a]; mine[1] = l[a]; }
+#pragma unroll
+                for (int b = 0; b < DVB; ++b)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mine[2 + b * 32 + 8 * (r >> 2) + 4 * half + (r & 3)] = o[a][b][r];
+            }
+        }
+        return;
+    }
     if (sink) {
         // the sink joins every map's sum as one more weight, exp(sink - maximum), with nothing to add to the output
         const float s2 = sink[hq] * 1.4426950408889634f;
@@ -276,6 +294,52 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     }      // the item's tiles
 }
 
+// The states of the workgroups that shared a token's keys (`part` [token, head, shares, map, 2 + VALUE_DIM]: maximum in
+// units of log 2, sum, output) added up in the order of the shares, then the sink, the difference of the maps and the
+// norm as above: one wave per (token, head).
+template <class T, int MAPS>
+__global__ __launch_bounds__(64) void diff_attn_merge_kernel(const float* __restrict__ part, T* __restrict__ out, int H,
+                                                             int S, int dv, float lambda, float out_eps, float out_scale,
+                                                             const float* __restrict__ sink) {
+    constexpr int W = 2 + VALUE_DIM, NV = (VALUE_DIM + 63) / 64;
+    const int64_t unit = blockIdx.x;
+    const int h = (int)(unit % H), lane = threadIdx.x;
+    float val[MAPS][NV];
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) {
+        const float* p = part + (unit * S * MAPS + a) * W;
+        float M = -INFINITY;
+        for (int s = 0; s < S; ++s) M = fmaxf(M, p[(int64_t)s * MAPS * W]);
+        const float s2 = sink ? sink[h] * 1.4426950408889634f : -INFINITY;
+        M = fmaxf(M, s2);
+        float L = sink ? __builtin_amdgcn_exp2f(s2 - M) : 0.f, O[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) O[v] = 0.f;
+        for (int s = 0; s < S; ++s) {
+            const float* q = p + (int64_t)s * MAPS * W;
+            if (q[0] == -INFINITY) continue;
+            const float f = __builtin_amdgcn_exp2f(q[0] - M);
+            L += q[1] * f;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) if (v * 64 + lane < VALUE_DIM) O[v] += q[2 + v * 64 + lane] * f;
+        }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) val[a][v] = O[v] / L;
+    }
+    float ss = 0.f, res[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        float x = val[0][v];
+        if (MAPS == 2) x -= lambda * val[MAPS - 1][v];
+        res[v] = v * 64 + lane < dv ? x : 0.f;
+        ss += res[v] * res[v];
+    }
+    ss = wave_sum(ss);
+    const float rr = out_eps >= 0.f ? out_scale / sqrtf(ss / (float)dv + out_eps) : out_scale;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) if (v * 64 + lane < dv) out[unit * dv + v * 64 + lane] = from_f32<T>(res[v] * rr);
+}
+
 extern "C" int li_diffattn_map_dim() { return MAP_DIM; }
 extern "C" int li_diffattn_value_dim() { return VALUE_DIM; }
 
@@ -285,7 +349,8 @@ extern "C" int li_diffattn_value_dim() { return VALUE_DIM; }
 extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages, const void* v_pages, int64_t page_stride,
                            const int* page_table, int max_pages, const int* pos, const int* tok_slot, const int* tile_t0,
                            const int* tile_n, int n_tiles, int H, int G, int maps, int dv, float scale, int block, int window,
-                           float lambda, float out_eps, float out_scale, const float* sink, hipStream_t stream) {
+                           float lambda, float out_eps, float out_scale, const float* sink, int key_shares, float* part,
+                           hipStream_t stream) {
     if (n_tiles <= 0) return LI_OK;
     if (H <= 0 || G <= 0 || H % G || dv <= 0 || dv > VALUE_DIM || block < 0 || window < 0) return LI_BAD_ARG;
     if (maps < 1 || maps > 2 || (dt != DT_F16 && dt != DT_BF16)) return LI_UNSUPPORTED;
@@ -297,7 +362,10 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
     const int heads = split ? 1 : (per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1));
     // a decode step with four or more query heads on a key/value head: the heads are a tile's columns
     const bool hc = split && per_kv >= 4;
-    dim3 grid(n_tiles, hc ? G * ((per_kv + 31) / 32) : H / heads);
+    // (then `key_shares` workgroups share a token's keys and leave their states in `part`, float32 [tokens, H, shares,
+    // maps, 2 + VALUE_DIM], for a second kernel)
+    const int shares = hc && key_shares > 1 && part ? key_shares : 1;
+    dim3 grid(n_tiles, hc ? G * ((per_kv + 31) / 32) : H / heads, shares);
     const int threads = split ? 256 : 64 * heads;
     const size_t lds = split ? (size_t)4 * maps * (hc ? 32 : 1) * (2 + VALUE_DIM) * sizeof(float) : 0;
 #define GO1(T, M, P, C)                                                                                                              \
@@ -307,7 +375,9 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
             hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)              \
             return LI_HIP_ERROR;                                                                                                     \
         kfn<<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, tile_n, H, G, dv, scale, block, window, \
-                                            lambda, out_eps, out_scale, split, sink);                                                \
+                                            lambda, out_eps, out_scale, split, sink, part);                                          \
+        if (shares > 1)                                                                                                              \
+            diff_attn_merge_kernel<T, M><<<n_tiles * H, 64, 0, stream>>>(part, (T*)out, H, shares, dv, lambda, out_eps, out_scale, sink); \
     } while (0)
 #define GO(T, M) do { if (hc) GO1(T, M, false, true); else if (split) GO1(T, M, false, false); else GO1(T, M, true, false); } while (0)
     if (dt == DT_F16) { if (maps == 1) GO(f16, 1); else GO(f16, 2); }

@@ -1253,14 +1253,16 @@ def diff_tiles(ctx, block=None, window=None):
 
 
 def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale, block, window, lam, out_eps, out_scale,
-                   out_dtype, tiles=None, sink=None) -> torch.Tensor:
+                   out_dtype, tiles=None, sink=None, key_shares: int = 1) -> torch.Tensor:
     """Attention of ``maps`` softmax maps (1 or 2) over the same values: o = a_1 - lam a_2, then (``out_eps`` not
     None) o divided by its root mean square over dv, times ``out_scale``.  A token at position p sees the keys
     from p - p % block on (``block`` 0: from 0; ``window`` w: at most the last w).  q [T, H, maps * DP] as
     ``qk_norm_store`` leaves it; returns [T, H * dv] in ``out_dtype``, the cache's type.  A float32 cache runs one
     workgroup per (token, head); a 16-bit cache runs on the matrix cores, one wave per (pair of tiles, head) with
     ``tiles`` from ``diff_tiles`` for the same block and window (None: every token an item of its own).
-    ``sink`` (float32 [H]): every map's sum of weights also counts exp(sink[head]), which has no key and no value."""
+    ``sink`` (float32 [H]): every map's sum of weights also counts exp(sink[head]), which has no key and no value.
+    ``key_shares`` (a decode step on the matrix cores with four or more query heads on a key/value head): that many
+    workgroups share a token's keys, and a second kernel adds up their states in order."""
     _dev(q, pos, tok_slot, sink)
     _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == n_heads), "sink: float32 [H]")
     t = q.shape[0]
@@ -1284,10 +1286,15 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
     if tiles is not None:
         _i32(tile_t0, 2 * n_tiles, "tile starts")
         _i32(tile_n, 2 * n_tiles, "tile sizes")
-    _check(_diffattn_lib(dp, (dv + 31) // 32 * 32).li_diffattn(
+    vd = (dv + 31) // 32 * 32
+    part = None
+    key_shares = max(1, min(int(key_shares), 64))
+    if tiles is None and key_shares > 1 and n_heads // n_kv_heads >= 4:
+        part = torch.empty((t, n_heads, key_shares, maps, 2 + vd), dtype=torch.float32, device=q.device)
+    _check(_diffattn_lib(dp, vd).li_diffattn(
         _ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
         page_table.shape[1], _ptr(pos), _ptr(tok_slot), _ptr(tile_t0), _ptr(tile_n), n_tiles, n_heads, n_kv_heads, maps, dv,
-        *tail), "diffattn")
+        *tail[:-1], key_shares if part is not None else 1, _ptr(part), tail[-1]), "diffattn")
     return out
 
 

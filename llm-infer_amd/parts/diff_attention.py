@@ -94,6 +94,15 @@ class DifferentialAttention(Part):
         return KVSpec(self.n_kv_heads, self.maps * ops.padded_map_dim(self.head_dim), self.window, self.v_head_dim, self.block,
                       "maps")
 
+    def _key_shares(self, ctx) -> int:
+        """Workgroups that share a token's keys in a decode step of a 16-bit model (a block bounds what a token sees)."""
+        if self.dtype == torch.float32 or not ctx.is_decode:
+            return 1
+        shares = ctx.decode_splits(self.n_kv_heads, self.n_heads)
+        if self.block:
+            shares = min(shares, max(1, self.block // 128))
+        return shares
+
     def forward(self, h, ctx, view, residual, owns_cache=True):
         if not owns_cache:
             raise ValueError("differential attention writes its own keys and values in every run")
@@ -103,5 +112,6 @@ class DifferentialAttention(Part):
         q = ops.qk_norm_store(proj, 0, self.q_norm, self.k_norm, self.qk_norm_eps, ctx.pos, ctx.tok_slot, kv, H, G, m, d, dv)
         a = ops.diff_attention(q, kv, ctx.pos, ctx.tok_slot, H, G, m, d, dv, self.scale, self.block, self.window, self.lam,
                                self.out_norm_eps, self.out_scale, self.dtype,
-                               ops.diff_tiles(ctx, self.block, self.window) if self.dtype != torch.float32 else None)
+                               ops.diff_tiles(ctx, self.block, self.window) if self.dtype != torch.float32 else None,
+                               key_shares=self._key_shares(ctx))
         ops.linear(a, self.wo, ops.EPI_ADD, out=residual)

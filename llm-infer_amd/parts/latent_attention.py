@@ -100,7 +100,8 @@ class LatentAttention(Part):
             q[:, :, :r].zero_()
         sixteen = self.dtype != torch.float32 and ops.diff_attention_fits(self.key_dim, r)
         a = ops.diff_attention(q, kv, ctx.pos, ctx.tok_slot, H, 1, 1, self.key_dim, r, self.scale, None, self.window, 0.0, None,
-                               1.0, self.dtype, ops.diff_tiles(ctx, None, self.window) if sixteen else None, sink=self.sinks)
+                               1.0, self.dtype, ops.diff_tiles(ctx, None, self.window) if sixteen else None, sink=self.sinks,
+                               key_shares=ctx.decode_splits(1, H) if sixteen and ctx.is_decode else 1)
         o = torch.empty((a.shape[0], H * dv), dtype=self.dtype, device=a.device)
         ops.head_linear(a, 0, r, self.w_uv, o, 0, dv, gate=proj if self.gate else None, gate_col=kv_col + r + rd)
         ops.linear(o, self.wo, ops.EPI_ADD, out=residual)
