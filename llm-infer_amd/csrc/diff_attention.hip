@@ -308,20 +308,20 @@ __global__ __launch_bounds__(64) void diff_attn_merge_kernel(const float* __rest
 #pragma unroll
     for (int a = 0; a < MAPS; ++a) {
         const float* p = part + (unit * S * MAPS + a) * W;
-        float M = -INFINITY;
-        for (int s = 0; s < S; ++s) M = fmaxf(M, p[(int64_t)s * MAPS * W]);
+        // lane s fetches share s's maximum and sum (S is at most 64), so no load waits for another
+        const float ms = lane < S ? p[(int64_t)lane * MAPS * W] : -INFINITY, ls = lane < S ? p[(int64_t)lane * MAPS * W + 1] : 0.f;
         const float s2 = sink ? sink[h] * 1.4426950408889634f : -INFINITY;
-        M = fmaxf(M, s2);
-        float L = sink ? __builtin_amdgcn_exp2f(s2 - M) : 0.f, O[NV];
+        const float M = fmaxf(wave_max(ms), s2);
+        const float fs = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
+        const float L = wave_sum(ls * fs) + (sink ? __builtin_amdgcn_exp2f(s2 - M) : 0.f);
+        float O[NV];
 #pragma unroll
         for (int v = 0; v < NV; ++v) O[v] = 0.f;
         for (int s = 0; s < S; ++s) {
-            const float* q = p + (int64_t)s * MAPS * W;
-            if (q[0] == -INFINITY) continue;
-            const float f = __builtin_amdgcn_exp2f(q[0] - M);
-            L += q[1] * f;
+            const float f = __shfl(fs, s, WAVE);
+            const float* q = p + (int64_t)s * MAPS * W + 2;
 #pragma unroll
-            for (int v = 0; v < NV; ++v) if (v * 64 + lane < VALUE_DIM) O[v] += q[2 + v * 64 + lane] * f;
+            for (int v = 0; v < NV; ++v) if (v * 64 + lane < VALUE_DIM) O[v] += q[v * 64 + lane] * f;
         }
 #pragma unroll
         for (int v = 0; v < NV; ++v) val[a][v] = O[v] / L;

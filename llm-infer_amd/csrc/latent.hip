@@ -205,9 +205,9 @@ extern "C" int li_latent_store(const float* proj, int stride, int q_col, int kv_
 // j < n_out.  Rows of `in` and `out` are addressed by a
 // stride per token and one per head, so that a head's part may lie inside a wider row.  `gate` not null: the result
 // is multiplied by sigmoid(gate[t][h * n_out + j]) (float32 rows, `gate_stride` apart).  Sums are float32.
-// head_linear_kernel (float32 models, and whatever the other does not take): a workgroup takes 16 tokens of one head,
+// head_linear_kernel (float32 models): a workgroup takes 16 tokens of one head,
 // their inputs wait in LDS and every thread owns outputs j.  head_linear_mfma_kernel (16-bit models): a wave owns 32
-// outputs x 32 tokens of one head, W^T as operand A and the tokens' inputs (rounded to the 16-bit type where they
+// outputs x up to 128 tokens of one head (a fragment of W serves four tiles of 32 tokens), W^T as operand A and the tokens' inputs (rounded to the 16-bit type where they
 // come in float32, as the sum of two such numbers) as operand B of the 32x32x16 matrix instruction, both read straight from memory, 16 bytes a lane
 // where n_in and the rows allow; the four waves of a workgroup take four blocks of outputs for the same tokens.
 // ---------------------------------------------------------------------------
@@ -247,6 +247,8 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TI* __restrict__
     }
 }
 
+#define HLM_TT 4            // tiles of 32 tokens that a wave multiplies with one fragment of W
+
 template <class TI, class T>
 __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const TI* __restrict__ in, int64_t in_st, int in_sh,
                                                                const T* __restrict__ W, T* __restrict__ out, int64_t out_st,
@@ -254,54 +256,72 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const TI* __restr
                                                                int n_tokens, int n_in, int n_out, int vec) {
     typedef typename Vec<T>::v8 v8;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
-    const int t = blockIdx.x * 32 + col, h = blockIdx.y, j0 = (blockIdx.z * 4 + wave) * 32;
+    const int tb = blockIdx.x * 32 * HLM_TT, h = blockIdx.y, j0 = (blockIdx.z * 4 + wave) * 32;
     if (j0 >= n_out) return;
-    const bool t_ok = t < n_tokens, j_ok = j0 + col < n_out;
+    const bool j_ok = j0 + col < n_out;
     const T* wrow = W + ((int64_t)h * n_out + (j_ok ? j0 + col : 0)) * n_in;
-    const TI* xrow = in + (int64_t)(t_ok ? t : 0) * in_st + (int64_t)h * in_sh;
-    f32x16 acc;
+    const int tiles = min(HLM_TT, (n_tokens - tb + 31) / 32);            // the same for all lanes
+    const TI* xrow[HLM_TT];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int u = 0; u < HLM_TT; ++u) xrow[u] = in + (int64_t)min(tb + 32 * u + col, n_tokens - 1) * in_st + (int64_t)h * in_sh;
+    f32x16 acc[HLM_TT];
+#pragma unroll
+    for (int u = 0; u < HLM_TT; ++u)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[u][r] = 0.f;
     for (int k0 = 0; k0 < n_in; k0 += 16) {
         const int i0 = k0 + 8 * half;
-        v8 a, b, b2;                     // b2: what the rounding of a float32 input leaves, so that the product sees 16 bits of it
-        float xf[8];
-        if (vec && i0 + 8 <= n_in) {
-            a = *(const v8*)(wrow + i0);
-            if (sizeof(TI) == 4) {
-                const f32x4 lo = *(const f32x4*)((const float*)xrow + i0), hi = *(const f32x4*)((const float*)xrow + i0 + 4);
+        const bool whole = vec && i0 + 8 <= n_in;
+        v8 a;
+        if (whole) a = *(const v8*)(wrow + i0);
+        else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { xf[e] = lo[e]; xf[4 + e] = hi[e]; }
-            } else {
-                b = *(const v8*)((const T*)xrow + i0);
-            }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                a[e] = i0 + e < n_in ? wrow[i0 + e] : from_f32<T>(0.f);
-                xf[e] = i0 + e < n_in ? to_f32(xrow[i0 + e]) : 0.f;
-                if (sizeof(TI) != 4) b[e] = from_f32<T>(xf[e]);
-            }
-        }
-        if (sizeof(TI) == 4) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) { b[e] = from_f32<T>(xf[e]); b2[e] = from_f32<T>(xf[e] - to_f32(b[e])); }
+            for (int e = 0; e < 8; ++e) a[e] = i0 + e < n_in ? wrow[i0 + e] : from_f32<T>(0.f);
         }
         if (!j_ok) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) a[e] = from_f32<T>(0.f);
         }
-        acc = mfma32(a, b, acc);
-        if (sizeof(TI) == 4) acc = mfma32(a, b2, acc);
-    }
-    if (!t_ok) return;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int j = j0 + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (j < n_out) {
-            float v = acc[r];
-            if (gate) v *= lt_sigmoid(gate[(int64_t)t * gate_st + (int64_t)h * n_out + j]);
-            out[(int64_t)t * out_st + (int64_t)h * out_sh + j] = from_f32<T>(v);
+        for (int u = 0; u < HLM_TT; ++u) {
+            if (u >= tiles) break;
+            v8 b, b2;                    // b2: what the rounding of a float32 input leaves, so that the product sees 16 bits of it
+            float xf[8];
+            if (whole) {
+                if (sizeof(TI) == 4) {
+                    const f32x4 lo = *(const f32x4*)((const float*)xrow[u] + i0), hi = *(const f32x4*)((const float*)xrow[u] + i0 + 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { xf[e] = lo[e]; xf[4 + e] = hi[e]; }
+                } else {
+                    b = *(const v8*)((const T*)xrow[u] + i0);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    xf[e] = i0 + e < n_in ? to_f32(xrow[u][i0 + e]) : 0.f;
+                    if (sizeof(TI) != 4) b[e] = from_f32<T>(xf[e]);
+                }
+            }
+            if (sizeof(TI) == 4) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { b[e] = from_f32<T>(xf[e]); b2[e] = from_f32<T>(xf[e] - to_f32(b[e])); }
+            }
+            acc[u] = mfma32(a, b, acc[u]);
+            if (sizeof(TI) == 4) acc[u] = mfma32(a, b2, acc[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < HLM_TT; ++u) {
+        const int t = tb + 32 * u + col;
+        if (u >= tiles || t >= n_tokens) continue;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int j = j0 + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (j < n_out) {
+                float v = acc[u][r];
+                if (gate) v *= lt_sigmoid(gate[(int64_t)t * gate_st + (int64_t)h * n_out + j]);
+                out[(int64_t)t * out_st + (int64_t)h * out_sh + j] = from_f32<T>(v);
+            }
         }
     }
 }
@@ -316,7 +336,7 @@ extern "C" int li_head_linear(const void* in, int in_dt, int64_t in_st, int in_s
         const int isz = in_dt == DT_F32 ? 4 : 2;
         const int vec = n_in % 8 == 0 && (uintptr_t)W % 16 == 0 && (uintptr_t)in % 16 == 0 && (in_st * isz) % 16 == 0 &&
                         ((int64_t)in_sh * isz) % 16 == 0;
-        dim3 grid((n_tokens + 31) / 32, H, (n_out + 127) / 128);
+        dim3 grid((n_tokens + 32 * HLM_TT - 1) / (32 * HLM_TT), H, (n_out + 127) / 128);
 #define GOM(TI, T) head_linear_mfma_kernel<TI, T><<<grid, 256, 0, stream>>>((const TI*)in, in_st, in_sh, (const T*)W, (T*)out, out_st, \
                                                                            out_sh, gate, gate_st, n_tokens, n_in, n_out, vec)
         if (in_dt == DT_F32) { if (w_dt == DT_F16) GOM(float, f16); else GOM(float, bf16); }
