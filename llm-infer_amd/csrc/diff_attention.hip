@@ -361,7 +361,8 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
     const int split = tile_t0 ? 0 : 1, per_kv = H / G;
     const int heads = split ? 1 : (per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1));
     // a decode step with four or more query heads on a key/value head: the heads are a tile's columns
-    const bool hc = split && per_kv >= 4;
+    // (where the 32 columns' states of four waves fit into the 160 KiB of LDS: two maps of wide values do not)
+    const bool hc = split && per_kv >= 4 && (size_t)4 * maps * 32 * (2 + VALUE_DIM) * sizeof(float) <= 150 * 1024;
     // (then `key_shares` workgroups share a token's keys and leave their states in `part`, float32 [tokens, H, shares,
     // maps, 2 + VALUE_DIM], for a second kernel)
     const int shares = hc && key_shares > 1 && part ? key_shares : 1;
