@@ -434,13 +434,17 @@ struct ScanSegments {
     float* seg_decay;           // [segments, H]
 };
 
-template <int NMAX, int PASS>
+// A head whose keys are more than 128 wide is shared by two waves a column block, 128 rows of S each (a lane's 256
+// registers of state would leave one wave a SIMD): RSPLIT = 2, and the two add their halves of y into rows that the
+// caller has cleared (two addends: the sum does not depend on their order).
+template <int NMAX, int NV, int RSPLIT, int PASS>
 __global__ __launch_bounds__(64) void mlstm_scan_kernel(
     const float* __restrict__ proj, int stride, int q_col, int k_col, int v_col, const float* __restrict__ coef,
     float qscale, float* __restrict__ S_state, const float* __restrict__ nm_state, float* __restrict__ nm_new,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart, const int* __restrict__ seq_qlen,
     float* __restrict__ y, int H, int d, int dv, ScanSegments sg) {
-    const int h = blockIdx.y, lane = threadIdx.x, col = blockIdx.z * 64 + lane;
+    const int h = blockIdx.y, lane = threadIdx.x, col = (blockIdx.z / RSPLIT) * 64 + lane;
+    const int r0 = (blockIdx.z % RSPLIT) * NMAX;             // this wave's first row of S
     const bool live = col < dv;
     int q0, n;
     float* S;
@@ -459,10 +463,9 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(
         nsrc = sg.seg_nrm + ((int64_t)seg * H + h) * d;
     }
     if (n <= 0) return;
-    constexpr int NV = (NMAX + 63) / 64;
     float s[NMAX], nl[NV];
 #pragma unroll
-    for (int i = 0; i < NMAX; ++i) s[i] = (PASS != 1 && live && i < d) ? S[(int64_t)i * dv] : 0.f;
+    for (int i = 0; i < NMAX; ++i) s[i] = (PASS != 1 && live && r0 + i < d) ? S[(int64_t)(r0 + i) * dv] : 0.f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) nl[v] = (PASS != 1 && v * 64 + lane < d) ? nsrc[v * 64 + lane] : 0.f;
     float qv[NV], kv[NV], x = 0.f, ca = 0.f, cb = 0.f, cm = 0.f, decay = 1.f;
@@ -490,22 +493,33 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(
 #pragma unroll
         for (int v = 0; v < NV; ++v) { nl[v] = a * nl[v] + b * kt[v]; nq += nl[v] * qt[v]; }
         if (PASS != 1) nq = wave_sum(nq);
+        // the registers that hold this wave's rows of k_t and q_t (the second half of them where the rows are shared)
+        constexpr int NH = (NMAX + 63) / 64;
+        float kh[NH], qh[NH];
+#pragma unroll
+        for (int v = 0; v < NH; ++v) {
+            kh[v] = (RSPLIT > 1 && r0) ? kt[(NV - NH + v) % NV] : kt[v];
+            qh[v] = (RSPLIT > 1 && r0) ? qt[(NV - NH + v) % NV] : qt[v];
+        }
         float acc = 0.f;
 #pragma unroll
         for (int i = 0; i < NMAX; ++i) {
-            const float kk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(kt[i >> 6]), i & 63));
+            const float kk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(kh[i >> 6]), i & 63));
+            float qq = 0.f;
+            if (PASS != 1) qq = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qh[i >> 6]), i & 63));
             s[i] = a * s[i] + kk * bx;
-            if (PASS != 1) {
-                const float qq = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qt[i >> 6]), i & 63));
-                acc += s[i] * qq;
-            }
+            if (PASS != 1) acc += s[i] * qq;
         }
-        if (PASS != 1 && live) y[(int64_t)(q0 + t) * H * dv + h * dv + col] = acc / (fmaxf(fabsf(nq), em) + 1e-6f);
+        if (PASS != 1 && live) {
+            float* to = y + (int64_t)(q0 + t) * H * dv + h * dv + col;
+            const float v = acc / (fmaxf(fabsf(nq), em) + 1e-6f);
+            if (RSPLIT > 1) atomicAdd(to, v); else *to = v;
+        }
     }
     if (PASS == 3) return;
     if (live) {
 #pragma unroll
-        for (int i = 0; i < NMAX; ++i) if (i < d) S[(int64_t)i * dv] = s[i];
+        for (int i = 0; i < NMAX; ++i) if (r0 + i < d) S[(int64_t)(r0 + i) * dv] = s[i];
     }
     if (blockIdx.z == 0) {
         float* to = PASS == 0 ? nm_new + ((int64_t)blockIdx.x * H + h) * (d + 1) : sg.seg_nrm + ((int64_t)blockIdx.x * H + h) * d;
@@ -545,16 +559,16 @@ __global__ void seg_combine_kernel(float* __restrict__ state, int64_t state_stri
     }
 }
 
-#define MLSTM_GO(NM, PASS, GRID) mlstm_scan_kernel<NM, PASS><<<GRID, 64, 0, stream>>>(proj, stride, q_col, k_col, v_col, coef, qscale, \
-        S_state, nm_state, nm_new, seq_slot, seq_qstart, seq_qlen, y, H, d, dv, sg)
-#define MLSTM_LAUNCH(PASS, GRID)                                                                             \
-    do {                                                                                                     \
-        if (d <= 16) MLSTM_GO(16, PASS, GRID); else if (d <= 32) MLSTM_GO(32, PASS, GRID);                   \
-        else if (d <= 64) MLSTM_GO(64, PASS, GRID); else if (d <= 128) MLSTM_GO(128, PASS, GRID);            \
-        else MLSTM_GO(256, PASS, GRID);                                                                      \
+#define MLSTM_GO(NM, NV, RS, PASS, GRID) mlstm_scan_kernel<NM, NV, RS, PASS><<<GRID, 64, 0, stream>>>(proj, stride, q_col, k_col, v_col, \
+        coef, qscale, S_state, nm_state, nm_new, seq_slot, seq_qstart, seq_qlen, y, H, d, dv, sg)
+#define MLSTM_LAUNCH(PASS, GRID)                                                                                       \
+    do {                                                                                                               \
+        if (d <= 16) MLSTM_GO(16, 1, 1, PASS, GRID); else if (d <= 32) MLSTM_GO(32, 1, 1, PASS, GRID);                 \
+        else if (d <= 64) MLSTM_GO(64, 1, 1, PASS, GRID); else if (d <= 128) MLSTM_GO(128, 2, 1, PASS, GRID);          \
+        else MLSTM_GO(128, 4, 2, PASS, GRID);                                                                          \
     } while (0)
 
-// coef: scratch float32 [T, H, 3]; nm_new: scratch float32 [sequences, H, d + 1].  n_segs > 0 (with the segment lists and
+// y must be cleared where d > 128 (two waves add their halves into it).  coef: scratch float32 [T, H, 3]; nm_new: scratch float32 [sequences, H, d + 1].  n_segs > 0 (with the segment lists and
 // scratch seg_S [segments, H, d, dv], seg_nrm [segments, H, d], seg_decay [segments, H]): the tokens run in segments.
 extern "C" int li_mlstm_scan(const float* proj, int stride, int q_col, int k_col, int v_col, int i_col, int f_col,
                              const float* i_bias, const float* f_bias, float cap, float qscale, float* S_state,
@@ -572,13 +586,13 @@ extern "C" int li_mlstm_scan(const float* proj, int stride, int q_col, int k_col
     ScanSegments sg{seg_seq, seg_t0, seg_n, seg_S, seg_nrm, seg_decay};
     if (n_segs <= 0) {
         if (!nm_new) return LI_BAD_ARG;
-        dim3 grid(n_seqs, H, (dv + 63) / 64);
+        dim3 grid(n_seqs, H, (dv + 63) / 64 * (d > 128 ? 2 : 1));
         MLSTM_LAUNCH(0, grid);
         mlstm_commit_kernel<<<dim3(n_seqs, H), 64, 0, stream>>>(nm_new, nm_state, seq_slot, seq_qlen, H, d);
     } else {
         if (!seq_qstart || !seq_qlen || !seg_seq || !seg_t0 || !seg_n || !seq_seg0 || !seq_nseg || !seg_S || !seg_nrm || !seg_decay)
             return LI_BAD_ARG;
-        dim3 grid(n_segs, H, (dv + 63) / 64);
+        dim3 grid(n_segs, H, (dv + 63) / 64 * (d > 128 ? 2 : 1));
         MLSTM_LAUNCH(1, grid);
         const int64_t per_head = (int64_t)d * dv;
         seg_combine_kernel<<<dim3(n_seqs, H, (unsigned)((per_head + 255) / 256)), 256, 0, stream>>>(

@@ -1647,7 +1647,8 @@ def mlstm_scan(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, q_s
           "mlstm normaliser state: float32 [slots, heads, d + 1]")
     seq_slot, qstart, qlen = _seq_arrays(ctx, t)
     dev = proj.device
-    y = torch.empty((t, heads * dv), dtype=torch.float32, device=dev)
+    # (keys more than 128 wide: two waves share a head's rows and add their halves of y)
+    y = (torch.zeros if d > 128 else torch.empty)((t, heads * dv), dtype=torch.float32, device=dev)
     coef = torch.empty((t, heads, 3), dtype=torch.float32, device=dev)
     fresh = seg = None
     if segments is None:
