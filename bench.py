@@ -178,7 +178,7 @@ def compare_configs(design: str, size: dict, layers: int, context: int) -> dict:
         stack = [{"type": kinds[i % 4], "mixer": mem if kinds[i % 4] == "mlstm" else lat,
                   "mlp": {"kind": "dense", "ff": size["ff"]} if i == 0 else routed} for i in range(layers)]
         other = {"architecture": "Dupolorn", "canon": {"taps": 3},
-                 "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 17}, "scale": 1.0}, "layers": stack,
+                 "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}, "scale": 1.0}, "layers": stack,
                  "logit_softcap": 30.0, "norm": {"eps": 1e-5}, "vocab": size["vocab"], "width": w, "max_positions": context}
         return {"llama": llama, design: other}
     assert design == "manirax"

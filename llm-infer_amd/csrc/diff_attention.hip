@@ -317,6 +317,7 @@ __global__ __launch_bounds__(64) void diff_attn_merge_kernel(const float* __rest
         float O[NV];
 #pragma unroll
         for (int v = 0; v < NV; ++v) O[v] = 0.f;
+#pragma unroll 4
         for (int s = 0; s < S; ++s) {
             const float f = __shfl(fs, s, WAVE);
             const float* q = p + (int64_t)s * MAPS * W + 2;

@@ -168,7 +168,8 @@ __global__ void latent_store_kernel(const float* __restrict__ proj, int stride, 
     T* kp = (T*)pg.k + (int64_t)page * pg.page_stride;
     T* vp = (T*)pg.v + (int64_t)page * pg.page_stride;
     const float fp = (float)p;
-    for (int i = threadIdx.x; i < KW; i += blockDim.x) {
+    // (few tokens: the grid's second dimension shares a token's key and heads among several workgroups)
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < KW; i += gridDim.y * blockDim.x) {
         float v = 0.f;
         if (i < r) {
             v = lat[i] * rr * norm_w[i];
@@ -179,7 +180,7 @@ __global__ void latent_store_kernel(const float* __restrict__ proj, int stride, 
         kp[k_offset(off, i, KW)] = from_f32<T>(v);
     }
     const int tail = KW - r;
-    for (int idx = threadIdx.x; idx < H * tail; idx += blockDim.x) {
+    for (int idx = blockIdx.y * blockDim.x + threadIdx.x; idx < H * tail; idx += gridDim.y * blockDim.x) {
         const int h = idx / tail, j = idx - h * tail;
         const float v = j < rd ? rotated(row + q_col + (int64_t)h * (d + rd) + d, j, rot, fp, freq) : 0.f;
         q_out[((int64_t)t * H + h) * KW + r + j] = from_f32<T>(v);
@@ -194,7 +195,8 @@ extern "C" int li_latent_store(const float* proj, int stride, int q_col, int kv_
     if (H <= 0 || d < 0 || rd < 0 || r <= 0 || rot < 0 || rot > rd || rot % 2) return LI_BAD_ARG;
     MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
     const int KW = round_up(r + rd, 16);
-    DISPATCH_T(dt, (latent_store_kernel<T><<<n, 256, 0, stream>>>(proj, stride, q_col, kv_col, norm_w, eps, freq, rot, pos,
+    dim3 grid(n, n >= 256 ? 1 : min(16, (max(KW, H * (KW - r)) + 255) / 256));
+    DISPATCH_T(dt, (latent_store_kernel<T><<<grid, 256, 0, stream>>>(proj, stride, q_col, kv_col, norm_w, eps, freq, rot, pos,
                                                                   tok_slot, (T*)q_out, pg, H, d, rd, r, KW)));
     LI_CHECK_LAUNCH();
     return LI_OK;

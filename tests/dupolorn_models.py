@@ -63,9 +63,9 @@ TINY_B = config(72, 97, [
 # 128 x 128 a head; one tap (the convolution is a weight on the input itself)
 TINY_C = config(256, 211, [
     layer(latent(8, 64, 64, 64, 192, second=True, base=10000.0), moe(4, 2, 96, shared=64)),
-    layer(mlstm(2, 128, 128, cap=12.0), dense(320)),
+    layer(mlstm(2, 128, 128, cap=11.0), dense(320)),
     layer(latent(4, 32, 16, 48, 320), dense(128)),
-], taps=1, eps=1e-5, scale=3.0, bigram=(509, 127, 17), softcap=30.0)
+], taps=1, eps=1e-5, scale=3.0, bigram=(509, 101, 13), softcap=25.0)
 
 ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 
