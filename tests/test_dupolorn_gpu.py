@@ -561,7 +561,26 @@ def test_trace_replay_in_three_schedules(lib, models, dtype, tmp_path):
 
 
 def test_command_line_reports_and_generates(lib, models):
-    folder, cfg, _ = models["A", "float32"]
+    folder, cfg, W = models["A", "float32"]
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    out = subprocess.run([sys.executable, os.path.join(root, "bin", "model_info"), folder], capture_output=True, text=True, timeout=300)
-    assert out.returncode == 0 and "Dupolorn" in out.stdout + out.stderr, out.stdout + out.stderr
+    prompts = [tokens(cfg, 9, 51), tokens(cfg, 2, 52)]
+    cmd = [sys.executable, os.path.join(root, "bin", "infer"), folder, "-n", "6", "-t", "0", "--dtype", "float32", "-T", "64"]
+    for p in prompts:
+        cmd += ["--tokens", ",".join(map(str, p))]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    got = [json.loads(line.split("tokens: ", 1)[1]) for line in res.stdout.splitlines() if " tokens: [" in line]
+    assert len(got) == 2
+    for p, new in zip(prompts, got):
+        toks = list(p)
+        for t in new:
+            last = P.forward(W, cfg, toks)[-1]
+            top2 = torch.topk(last, 2).values
+            if (top2[0] - top2[1]).item() > 1e-3:
+                assert t == int(last.argmax())
+            toks.append(t)
+    for word in ("Dimensions: 96", "Vocab size: 131"):
+        assert word in res.stdout, res.stdout
+    info = subprocess.run([sys.executable, os.path.join(root, "bin", "model_info"), folder], capture_output=True, text=True,
+                          timeout=300)
+    assert info.returncode == 0 and "Architecture: Dupolorn" in info.stdout and "The tensors fit the model." in info.stdout
