@@ -328,17 +328,19 @@ def test_latent_attention_finds_a_far_key_and_feels_its_sink(lib, dtype):
     assert error(got["a"], ref2) < TOL[dtype]
 
 
-def test_decoding_far_into_a_context_with_many_heads(lib):
-    """Eight heads on the one latent and a context of ten pages: a 16-bit decode step then takes the heads as the
-    columns of one tile and lets several workgroups share a token's keys; two requests of unequal length together."""
+@pytest.mark.parametrize("H, na, nb", [(8, 660, 200), (40, 330, 90)])
+def test_decoding_far_into_a_context_with_many_heads(lib, H, na, nb):
+    """Many heads on the one latent and a context of several pages: a 16-bit decode step then takes the heads as the
+    columns of a tile (forty heads: two tiles) and lets several workgroups share a token's keys; two requests of unequal
+    length together."""
     width = 64
-    mixer = M.latent(8, 16, 16, 24, 48, second=True, base=1000.0)
+    mixer = M.latent(H, 16, 16, 24, 48, second=True, base=1000.0)
     cfg = one_layer(mixer, width=width)
     g = torch.Generator().manual_seed(17)
     W = M.mixer_weights(mixer[0], mixer[1], width, g, torch.bfloat16, sharp=2.0)
     part = build_mixer(inner_spec(cfg), W, "bfloat16", cfg._position(cfg.layers[0]))
-    h_of = {"a": torch.randn(660, width, generator=g).bfloat16().float(), "b": torch.randn(200, width, generator=g).bfloat16().float()}
-    got, _ = run_mixer(part, h_of, [{"a": 620, "b": 160}] + [{"a": 1, "b": 1}] * 40, "bfloat16")
+    h_of = {"a": torch.randn(na, width, generator=g).bfloat16().float(), "b": torch.randn(nb, width, generator=g).bfloat16().float()}
+    got, _ = run_mixer(part, h_of, [{"a": na - 40, "b": nb - 40}] + [{"a": 1, "b": 1}] * 40, "bfloat16")
     for r, h in h_of.items():
         ref = P.latent_attention(h.double(), M.widen(W), mixer[1], 1e-5, True)
         tol = max(TOL["bfloat16"], 3 * error(P.latent_attention(h.double(), M.widen(W), mixer[1], 1e-5, True, store=torch.bfloat16), ref))
