@@ -3,7 +3,7 @@
     engine = llm_infer_amd.load("model_dir", max_tokens=65536)
     new_tokens = engine.generate([[1, 2, 3], [4, 5]], max_new_tokens=16, temperature=0.0)
 """
-from .config import ConfigError, DupolornConfig, LlamaConfig, ManiraxConfig, RisonexConfig
+from .config import ConfigError, DupolornConfig, FavizenConfig, LlamaConfig, ManiraxConfig, RisonexConfig
 from .tensor import Tensor
 from .registry import (config_from_dict, config_from_folder, register_architecture, register_block,
                        register_embedding, register_feed_forward, register_head, register_mixer,
@@ -15,6 +15,7 @@ register_architecture("LlamaForCausalLM", LlamaConfig)
 register_architecture("Manirax", ManiraxConfig)
 register_architecture("Risonex", RisonexConfig)
 register_architecture("Dupolorn", DupolornConfig)
+register_architecture("Favizen", FavizenConfig)
 
 
 def load(folder: str, dtype: str | None = None, max_tokens: int = 8192, n_slots=None, kv_round=None):

@@ -11,7 +11,9 @@
 // page holds the values.  A weight enters the second product as the sum of two 16-bit numbers (its rounding and the
 // rounding of the remainder), so that the product sees 16 bits of it.  At the end o = O_1 / l_1 - lambda O_2 / l_2,
 // divided by its root mean square over the value size and multiplied by out_scale.  `sink` not null: every map's sum
-// of weights also counts exp(sink[head]), a score with no key and no value that is not scaled.
+// of weights also counts exp(sink[head]), a score with no key and no value that is not scaled.  `slopes` not null:
+// the score of the key at position j loses slopes[head] * (p - j), the sink nothing.  `gate` not null: a head's output
+// is multiplied by the sigmoid of gate[token][gate_col + head] (float32 rows of gate_stride numbers).
 #include "common.h"
 
 #ifndef MAP_DIM
@@ -38,7 +40,8 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, const int* __restrict__ tile_t0, const int* __restrict__ tile_n, int H, int G,
     int dv, float scale, int block, int window, float lambda, float out_eps, float out_scale, int split,
-    const float* __restrict__ sink, float* __restrict__ shares_out) {
+    const float* __restrict__ sink, float* __restrict__ shares_out, const float* __restrict__ slopes,
+    const float* __restrict__ gate, int gate_stride, int gate_col) {
     typedef typename Vec<T>::v8 v8;
     constexpr int D16 = MAP_DIM / 16, KW = MAPS * MAP_DIM, DVB = VALUE_DIM / 32;
     extern __shared__ float lds[];
@@ -80,6 +83,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     if (window > 0) lo_last = max(lo_last, p_last - window + 1);
     const bool whole_tile = n == 32;
     const float scale2 = scale * 1.4426950408889634f;
+    const float slope2 = slopes ? slopes[hq] * 1.4426950408889634f : 0.f;      // what a score loses for every position of distance
     const int* table = pg.page_table + (int64_t)tok_slot[t0] * pg.max_pages;
 
     v8 qf[MAPS][D16];
@@ -143,14 +147,23 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
             // sees need no mask
             float tmax = -INFINITY;
             if (whole_tile && kt * 32 >= lo_last && kt * 32 + 31 <= p0) {
+                if (slopes) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) { acc[r] *= scale2; tmax = fmaxf(tmax, acc[r]); }
+                    for (int r = 0; r < 16; ++r) {
+                        const int key = kt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        acc[r] = acc[r] * scale2 - slope2 * (float)(pq - key);
+                        tmax = fmaxf(tmax, acc[r]);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) { acc[r] *= scale2; tmax = fmaxf(tmax, acc[r]); }
+                }
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = kt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
                     const bool seen = has_query && key >= lo_q && key <= pq;
-                    acc[r] = seen ? acc[r] * scale2 : -INFINITY;
+                    acc[r] = seen ? acc[r] * scale2 - slope2 * (float)(pq - key) : -INFINITY;
                     tmax = fmaxf(tmax, acc[r]);
                 }
             }
@@ -280,7 +293,9 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
             ss += v * v;
         }
     ss += __shfl_xor(ss, 32, WAVE);
-    const float rr = out_eps >= 0.f ? out_scale / sqrtf(ss / (float)dv + out_eps) : out_scale;
+    float rr = out_eps >= 0.f ? out_scale / sqrtf(ss / (float)dv + out_eps) : out_scale;
+    if (gate && has_query)             // one number a (token, head)
+        rr *= 1.f / (1.f + expf(-gate[(int64_t)(t0 + (HC ? 0 : col)) * gate_stride + gate_col + hq]));
     if (has_query) {
         T* orow = out + ((int64_t)(t0 + (HC ? 0 : col)) * H + hq) * dv;
 #pragma unroll
@@ -300,7 +315,8 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
 template <class T, int MAPS>
 __global__ __launch_bounds__(64) void diff_attn_merge_kernel(const float* __restrict__ part, T* __restrict__ out, int H,
                                                              int S, int dv, float lambda, float out_eps, float out_scale,
-                                                             const float* __restrict__ sink) {
+                                                             const float* __restrict__ sink, const float* __restrict__ gate,
+                                                             int gate_stride, int gate_col) {
     constexpr int W = 2 + VALUE_DIM, NV = (VALUE_DIM + 63) / 64;
     const int64_t unit = blockIdx.x;
     const int h = (int)(unit % H), lane = threadIdx.x;
@@ -336,7 +352,8 @@ __global__ __launch_bounds__(64) void diff_attn_merge_kernel(const float* __rest
         ss += res[v] * res[v];
     }
     ss = wave_sum(ss);
-    const float rr = out_eps >= 0.f ? out_scale / sqrtf(ss / (float)dv + out_eps) : out_scale;
+    float rr = out_eps >= 0.f ? out_scale / sqrtf(ss / (float)dv + out_eps) : out_scale;
+    if (gate) rr *= 1.f / (1.f + expf(-gate[(unit / H) * gate_stride + gate_col + h]));
 #pragma unroll
     for (int v = 0; v < NV; ++v) if (v * 64 + lane < dv) out[unit * dv + v * 64 + lane] = from_f32<T>(res[v] * rr);
 }
@@ -351,8 +368,9 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
                            const int* page_table, int max_pages, const int* pos, const int* tok_slot, const int* tile_t0,
                            const int* tile_n, int n_tiles, int H, int G, int maps, int dv, float scale, int block, int window,
                            float lambda, float out_eps, float out_scale, const float* sink, int key_shares, float* part,
-                           hipStream_t stream) {
+                           const float* slopes, const float* gate, int gate_stride, int gate_col, hipStream_t stream) {
     if (n_tiles <= 0) return LI_OK;
+    if (gate && (gate_col < 0 || gate_col + H > gate_stride)) return LI_BAD_ARG;
     if (H <= 0 || G <= 0 || H % G || dv <= 0 || dv > VALUE_DIM || block < 0 || window < 0) return LI_BAD_ARG;
     if (maps < 1 || maps > 2 || (dt != DT_F16 && dt != DT_BF16)) return LI_UNSUPPORTED;
     if ((tile_t0 == nullptr) != (tile_n == nullptr)) return LI_BAD_ARG;
@@ -377,9 +395,10 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
             hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)              \
             return LI_HIP_ERROR;                                                                                                     \
         kfn<<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, tile_n, H, G, dv, scale, block, window, \
-                                            lambda, out_eps, out_scale, split, sink, part);                                          \
+                                            lambda, out_eps, out_scale, split, sink, part, slopes, gate, gate_stride, gate_col);     \
         if (shares > 1)                                                                                                              \
-            diff_attn_merge_kernel<T, M><<<n_tiles * H, 64, 0, stream>>>(part, (T*)out, H, shares, dv, lambda, out_eps, out_scale, sink); \
+            diff_attn_merge_kernel<T, M><<<n_tiles * H, 64, 0, stream>>>(part, (T*)out, H, shares, dv, lambda, out_eps, out_scale, sink, \
+                                                                      gate, gate_stride, gate_col);                                  \
     } while (0)
 #define GO(T, M) do { if (hc) GO1(T, M, false, true); else if (split) GO1(T, M, false, false); else GO1(T, M, true, false); } while (0)
     if (dt == DT_F16) { if (maps == 1) GO(f16, 1); else GO(f16, 2); }

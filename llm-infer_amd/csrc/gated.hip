@@ -1,0 +1,252 @@
+// Kernels of decoders whose sub-layers stand between two norms and whose softmax attention carries a sink, a gate
+// per head and either a rotation of half-paired dimensions or a bias by distance: a bias added to the columns of a
+// product's float32 rows, the rotation of q and k with the write of keys and values into the paged cache, the norm
+// of a sub-layer's output added into the residual stream, the clamped gated activation of a feed-forward (with a
+// bias and with the experts' routing weights), and the routing weights of experts that a table assigns to token ids.
+// The attention itself is hybrid.hip's (float32) and diff_attention.hip's (matrix cores).  Every size is a run-time
+// value; norms, angles and the residual sum are float32 whatever the type of the matrices.
+#include "common.h"
+
+#define DISPATCH_T(dt, CALL)                                     \
+    do {                                                         \
+        if ((dt) == DT_F32) { typedef float T; CALL; }           \
+        else if ((dt) == DT_F16) { typedef f16 T; CALL; }        \
+        else if ((dt) == DT_BF16) { typedef bf16 T; CALL; }      \
+        else return LI_BAD_ARG;                                  \
+    } while (0)
+
+// ---------------------------------------------------------------------------
+// rows[t][col0 + i] += b[i] for i < n: the bias of a product whose kernel has none.
+// ---------------------------------------------------------------------------
+__global__ void add_bias_kernel(float* __restrict__ rows, int stride, int col0, const float* __restrict__ b, int n) {
+    float* row = rows + (int64_t)blockIdx.x * stride + col0;
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < n; i += gridDim.y * blockDim.x) row[i] += b[i];
+}
+
+extern "C" int li_add_bias(float* rows, int stride, int col0, const float* b, int n_rows, int n, hipStream_t stream) {
+    if (n_rows <= 0 || n <= 0) return LI_OK;
+    if (col0 < 0 || col0 + n > stride) return LI_BAD_ARG;
+    dim3 grid(n_rows, n_rows >= 1024 ? 1 : (n + 1023) / 1024);
+    add_bias_kernel<<<grid, 256, 0, stream>>>(rows, stride, col0, b, n);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// x[i] *= s for n float32 numbers (a model's logits times a constant).
+__global__ void scale_values_kernel(float* __restrict__ x, int64_t n, float s) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) x[i] *= s;
+}
+
+extern "C" int li_scale_values(float* x, int64_t n, float s, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    scale_values_kernel<<<blocks, 256, 0, stream>>>(x, n, s);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// From float32 rows that hold a token's q heads [H, d] from column q_col, its k heads [G, d] from k_col and its
+// values [G, dv] from v_col (v_col may be k_col: the values are the keys as projected): q and k are turned by the
+// token's position p in their first `rot` dimensions, dimension i paired with i + rot / 2,
+//   (u, v) -> (u cos a - v sin a, v cos a + u sin a),  a = p * inv_freq[i]   (float32 angles, accurate sin and cos),
+// the values are not.  q goes to q_out [T, H, DP] in the cache's type (DP = d rounded up to 16, zeros behind d),
+// k (padded likewise) and v into the page of position p in matrix-operand order (common.h; one map of keys).
+// G_store 0: only q (a layer that reads another layer's keys and values).
+// ---------------------------------------------------------------------------
+struct StorePages {
+    void* k;
+    void* v;
+    int64_t page_stride;
+    const int* page_table;
+    int max_pages;
+};
+
+template <class T>
+__global__ void rot_store_kernel(const float* __restrict__ rows, int stride, int q_col, int k_col, int v_col,
+                                 const float* __restrict__ inv_freq, int rot, const int* __restrict__ pos,
+                                 const int* __restrict__ tok_slot, T* __restrict__ q_out, StorePages pg, int H, int G,
+                                 int d, int dv) {
+    const int t = blockIdx.x, p = pos[t], DP = round_up(d, 16), half = rot >> 1;
+    const float* row = rows + (int64_t)t * stride;
+    T* kp = nullptr;
+    T* vp = nullptr;
+    const int off = p % PAGE;
+    if (G > 0) {
+        const int page = pg.page_table[(int64_t)tok_slot[t] * pg.max_pages + p / PAGE];
+        kp = (T*)pg.k + (int64_t)page * pg.page_stride;
+        vp = (T*)pg.v + (int64_t)page * pg.page_stride;
+    }
+    const int n_qk = (H + G) * DP, total = n_qk + G * dv;
+    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < total; e += gridDim.y * blockDim.x) {
+        if (e < n_qk) {
+            const int u = e / DP, i = e - u * DP;
+            const bool is_q = u < H;
+            const float* src = row + (is_q ? q_col + u * d : k_col + (u - H) * d);
+            float val = 0.f;
+            if (i < d) {
+                val = src[i];
+                if (i < rot) {
+                    const int j = i < half ? i : i - half;
+                    float sn, cs;
+                    sincosf((float)p * inv_freq[j], &sn, &cs);
+                    val = i < half ? val * cs - src[i + half] * sn : val * cs + src[i - half] * sn;
+                }
+            }
+            if (is_q) q_out[((int64_t)t * H + u) * DP + i] = from_f32<T>(val);
+            else kp[(int64_t)(u - H) * k_head_elems(DP) + k_offset(off, i, DP)] = from_f32<T>(val);
+        } else {
+            const int r = e - n_qk, g = r / dv, j = r - g * dv;
+            vp[(int64_t)g * v_head_elems(dv) + v_offset(off, j, dv)] = from_f32<T>(row[v_col + r]);
+        }
+    }
+}
+
+extern "C" int li_rot_store(const float* rows, int stride, int q_col, int k_col, int v_col, const float* inv_freq, int rot,
+                            const int* pos, const int* tok_slot, void* q_out, void* k_pages, void* v_pages,
+                            int64_t page_stride, const int* page_table, int max_pages, int dt, int n, int H, int G_store,
+                            int d, int dv, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (H <= 0 || G_store < 0 || d <= 0 || dv <= 0 || rot < 0 || rot > d || (rot & 1) || (rot && !inv_freq)) return LI_BAD_ARG;
+    if (q_col < 0 || q_col + H * d > stride) return LI_BAD_ARG;
+    if (G_store && (k_col < 0 || v_col < 0 || k_col + G_store * d > stride || v_col + G_store * dv > stride)) return LI_BAD_ARG;
+    StorePages pg{k_pages, v_pages, page_stride, page_table, max_pages};
+    const int total = (H + G_store) * round_up(d, 16) + G_store * dv;
+    dim3 grid(n, n >= 512 ? 1 : (total + 255) / 256);
+    DISPATCH_T(dt, (rot_store_kernel<T><<<grid, 256, 0, stream>>>(rows, stride, q_col, k_col, v_col, inv_freq, rot, pos, tok_slot,
+                                                              (T*)q_out, pg, H, G_store, d, dv)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// x[t] += (y[t] + b) / sqrt(mean((y[t] + b)^2) + eps) * w: the norm on a sub-layer's output and the residual sum in
+// one pass over the row (b may be null).  One workgroup a row; the row stays in registers up to 8,192 elements.
+// ---------------------------------------------------------------------------
+#define RA_THREADS 256
+#define RA_KEEP 8          // 4 elements x RA_KEEP x RA_THREADS = 8,192 elements kept
+
+__global__ __launch_bounds__(RA_THREADS) void rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                                 const float* __restrict__ b, const float* __restrict__ w,
+                                                                 float eps, int width) {
+    __shared__ float scratch[16];
+    const int64_t row = blockIdx.x;
+    const float* yr = y + row * width;
+    float* xr = x + row * width;
+    float ss = 0.f;
+    if ((width & 3) == 0 && width <= 4 * RA_KEEP * RA_THREADS) {
+        f32x4 keep[RA_KEEP];
+        const int quads = width >> 2;
+#pragma unroll
+        for (int c = 0; c < RA_KEEP; ++c) {
+            const int i = threadIdx.x + c * RA_THREADS;
+            if (i < quads) {
+                f32x4 v = *(const f32x4*)(yr + 4 * i);
+                if (b) { const f32x4 bb = *(const f32x4*)(b + 4 * i); v[0] += bb[0]; v[1] += bb[1]; v[2] += bb[2]; v[3] += bb[3]; }
+                keep[c] = v;
+                ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+            }
+        }
+        const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+#pragma unroll
+        for (int c = 0; c < RA_KEEP; ++c) {
+            const int i = threadIdx.x + c * RA_THREADS;
+            if (i < quads) {
+                const f32x4 ww = *(const f32x4*)(w + 4 * i);
+                f32x4 o = *(f32x4*)(xr + 4 * i);
+                o[0] += keep[c][0] * r * ww[0]; o[1] += keep[c][1] * r * ww[1];
+                o[2] += keep[c][2] * r * ww[2]; o[3] += keep[c][3] * r * ww[3];
+                *(f32x4*)(xr + 4 * i) = o;
+            }
+        }
+        return;
+    }
+    for (int i = threadIdx.x; i < width; i += RA_THREADS) { const float v = yr[i] + (b ? b[i] : 0.f); ss += v * v; }
+    const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += RA_THREADS) xr[i] += (yr[i] + (b ? b[i] : 0.f)) * r * w[i];
+}
+
+extern "C" int li_rmsnorm_add(float* x, const float* y, const float* b, const float* w, float eps, int n_rows, int width,
+                              hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (width <= 0 || !x || !y || !w) return LI_BAD_ARG;
+    rmsnorm_add_kernel<<<n_rows, RA_THREADS, 0, stream>>>(x, y, b, w, eps, width);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The clamped gated activation on the float32 sums of a product over interleaved rows (column 2j: gate j, column
+// 2j + 1: up j), z [T, 2 F] with F = n_blocks * ff + tail:
+//   g = min(gate + b_gate, limit),  u = clamp(up + b_up, -limit, limit),  out[t][j] = g sigmoid(alpha g) (u + shift)
+// `bias` (float32 [2 F], interleaved as z is) may be null.  The last `tail` outputs take tail_limit.  `weights` not
+// null (float32 [T, n_blocks (+ 1 with a tail)]): block e of a row (an expert's hidden row) is multiplied by
+// weights[t][e], the tail by weights[t][n_blocks]; a weight of 0 writes 0 whatever the sums hold.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float clamped_glu_(float g, float u, float limit, float alpha, float shift) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-alpha * g)) * (u + shift);
+}
+
+template <class T>
+__global__ void clamped_glu_kernel(const float* __restrict__ z, const float* __restrict__ bias, T* __restrict__ out,
+                                   int n_blocks, int ff, int tail, float limit, float tail_limit, float alpha, float shift,
+                                   const float* __restrict__ weights) {
+    const int64_t row = blockIdx.x;
+    const int F = n_blocks * ff + tail, wcols = n_blocks + (tail ? 1 : 0);
+    const float* zr = z + row * 2 * F;
+    for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < F; j += gridDim.y * blockDim.x) {
+        const bool in_tail = j >= n_blocks * ff;
+        float w = 1.f;
+        if (weights) w = weights[row * wcols + (in_tail ? n_blocks : j / ff)];
+        float o = 0.f;
+        if (w != 0.f) {
+            const f32x2 gu = *(const f32x2*)(zr + 2 * j);
+            const float g = gu[0] + (bias ? bias[2 * j] : 0.f), u = gu[1] + (bias ? bias[2 * j + 1] : 0.f);
+            o = clamped_glu_(g, u, in_tail ? tail_limit : limit, alpha, shift) * w;
+        }
+        out[row * F + j] = from_f32<T>(o);
+    }
+}
+
+extern "C" int li_clamped_glu(const float* z, const float* bias, void* out, int dt, int n_rows, int n_blocks, int ff, int tail,
+                              float limit, float tail_limit, float alpha, float shift, const float* weights,
+                              hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (n_blocks < 0 || ff < 0 || tail < 0 || n_blocks * ff + tail <= 0) return LI_BAD_ARG;
+    const int F = n_blocks * ff + tail;
+    dim3 grid(n_rows, n_rows >= 1024 ? 1 : (F + 1023) / 1024);
+    DISPATCH_T(dt, (clamped_glu_kernel<T><<<grid, 256, 0, stream>>>(z, bias, (T*)out, n_blocks, ff, tail, limit, tail_limit, alpha,
+                                                                shift, weights)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Experts by table: row table[token] [top] names the experts of a token (they differ), each with weight 1 / top.
+// weights [T, wcols] gets the dense row (0 where not named); with has_gate 1 its last column is the sigmoid of the
+// token's gate logit (float32 [T]) for an expert that every token uses, with has_gate 2 it is 1.
+// ---------------------------------------------------------------------------
+__global__ void table_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table, int top, int n_experts,
+                                   const float* __restrict__ gate_logits, int has_gate, float* __restrict__ weights) {
+    const int64_t t = blockIdx.x;
+    const int wcols = n_experts + (has_gate ? 1 : 0);
+    float* w = weights + t * wcols;
+    const int* mine = table + (int64_t)tokens[t] * top;
+    for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+        float v = 0.f;
+        for (int k = 0; k < top; ++k) if (mine[k] == e) v = 1.f / (float)top;
+        w[e] = v;
+    }
+    if (has_gate && threadIdx.x == 0) w[n_experts] = has_gate == 2 ? 1.f : 1.f / (1.f + expf(-gate_logits[t]));
+}
+
+extern "C" int li_table_route(const int* tokens, const int* table, int top, int n_experts, const float* gate_logits,
+                              int has_gate, float* weights, int n, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (top < 1 || n_experts < 1 || top > n_experts || has_gate < 0 || has_gate > 2 || (has_gate == 1 && !gate_logits)) return LI_BAD_ARG;
+    table_route_kernel<<<n, 64, 0, stream>>>(tokens, table, top, n_experts, gate_logits, has_gate, weights);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

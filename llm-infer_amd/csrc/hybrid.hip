@@ -165,7 +165,9 @@ extern "C" int li_qk_norm_store(const float* qkv, int stride, int col0, const fl
 // least p - w + 1).  Each of `maps` (1 or 2) maps is a softmax of its own over scores q_m . k_m * scale; with a_m
 // the maps' weighted sums of the SAME values,  o = a_1 - lambda a_2  (one map: o = a_1).  out_eps >= 0: o is
 // divided by its root mean square over dv and multiplied by out_scale.  `sink` not null: every map's sum of weights
-// also counts exp(sink[head]), a score with no key and no value that is not scaled.  Scores, weights, sums: float32.
+// also counts exp(sink[head]), a score with no key and no value that is not scaled.  `slopes` not null: the score of
+// the key at position j loses slopes[head] * (p - j) (the sink loses nothing).  `gate` not null: the head's output is
+// multiplied by the sigmoid of gate[t][gate_col + head] (float32 rows of gate_stride numbers).  Scores, weights, sums: float32.
 // The waves of the workgroup take the tiles of 64 keys in turn, a lane a key; each keeps a running maximum and
 // sum per map (online softmax) and its share of the output, and the shares are merged through LDS in wave order.
 // ---------------------------------------------------------------------------
@@ -176,7 +178,8 @@ template <class T, int MAPS>
 __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, int H, int G, int d, int dv, float scale, int block, int window, float lambda,
-    float out_eps, float out_scale, const float* __restrict__ sink) {
+    float out_eps, float out_scale, const float* __restrict__ sink, const float* __restrict__ slopes,
+    const float* __restrict__ gate, int gate_stride, int gate_col) {
     extern __shared__ float lds[];
     const int DP = round_up(d, 16), KW = MAPS * DP;
     float* sq = lds;                                   // [KW]
@@ -186,6 +189,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
     __shared__ float scratch[16];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = h / (H / G), p = pos[t];
+    const float slope = slopes ? slopes[h] : 0.f;      // a score loses slope * (distance to its key)
     int lo = block > 0 ? p - p % block : 0;
     if (window > 0) lo = max(lo, p - window + 1);
     for (int i = threadIdx.x; i < KW; i += blockDim.x) sq[i] = to_f32(q[((int64_t)t * H + h) * KW + i]);
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
         for (int a = 0; a < MAPS; ++a) {
             float acc = 0.f;
             if (kh) for (int i = 0; i < d; ++i) acc += sq[a * DP + i] * to_f32(kh[k_offset(j % PAGE, a * DP + i, KW)]);
-            s[a] = kh ? acc * scale : -INFINITY;
+            s[a] = kh ? acc * scale - slope * (float)(p - j) : -INFINITY;
         }
         float pw[MAPS];
 #pragma unroll
@@ -281,6 +285,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
     }
     float r = out_scale;
     if (out_eps >= 0.f) r = out_scale / sqrtf(block_sum(ss, scratch) / (float)dv + out_eps);   // waves 1.. add 0
+    if (gate) r *= sigmoidf_(gate[(int64_t)t * gate_stride + gate_col + h]);                   // one number a head
     if (wave == 0) {
 #pragma unroll
         for (int c = 0; c < DA_MAXV; ++c) {
@@ -293,16 +298,19 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
 extern "C" int li_diff_attn(const void* q, void* out, int dt, void* k_pages, void* v_pages, int64_t page_stride,
                             const int* page_table, int max_pages, const int* pos, const int* tok_slot, int n, int H, int G,
                             int maps, int d, int dv, float scale, int block, int window, float lambda, float out_eps,
-                            float out_scale, const float* sink, hipStream_t stream) {
+                            float out_scale, const float* sink, const float* slopes, const float* gate, int gate_stride,
+                            int gate_col, hipStream_t stream) {
     if (n <= 0) return LI_OK;
     if (H <= 0 || G <= 0 || H % G || d <= 0 || dv <= 0 || block < 0 || window < 0) return LI_BAD_ARG;
+    if (gate && (gate_col < 0 || gate_col + H > gate_stride)) return LI_BAD_ARG;
     if (maps < 1 || maps > 2 || dv > 64 * DA_MAXV) return LI_UNSUPPORTED;
     MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
     dim3 grid(n, H), blk(64 * DA_WAVES);
     const size_t lds = (size_t)(maps * round_up(d, 16) + 2 * DA_WAVES * maps + DA_WAVES * maps * dv) * sizeof(float);
     if (lds > 60000) return LI_UNSUPPORTED;
 #define GO(M) diff_attn_kernel<T, M><<<grid, blk, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, H, G, d, dv, scale, \
-                                                                 block, window, lambda, out_eps, out_scale, sink)
+                                                                 block, window, lambda, out_eps, out_scale, sink, slopes, gate, \
+                                                                 gate_stride, gate_col)
     DISPATCH_T(dt, { if (maps == 1) GO(1); else GO(2); });
 #undef GO
     LI_CHECK_LAUNCH();
@@ -384,6 +392,24 @@ extern "C" int li_conv_add(const float* in, int stride, int col0, const float* w
     dim3 cgrid(n_tokens, (channels + 255) / 256);
     DISPATCH_T(dt, (conv_silu_kernel<T, false, true><<<cgrid, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, (T*)out,
                                                                                 channels, taps)));
+    if (taps > 1) {
+        dim3 grid(n_seqs, (channels + 255) / 256);
+        conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);
+    }
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// The same convolution alone: no activation, the input not added, float32 out (what a mixer convolves behind its own
+// input product before anything else is done to it).
+extern "C" int li_conv_plain(const float* in, int stride, int col0, const float* w, const float* b, float* hist,
+                             const int* pos, const int* tok_slot, const int* seq_slot, const int* seq_qstart,
+                             const int* seq_qlen, float* out, int n_tokens, int n_seqs, int channels, int taps,
+                             hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (channels <= 0 || taps < 1 || taps > CONV_MAX_TAPS) return LI_BAD_ARG;
+    dim3 cgrid(n_tokens, (channels + 255) / 256);
+    conv_silu_kernel<float, false, false><<<cgrid, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, out, channels, taps);
     if (taps > 1) {
         dim3 grid(n_seqs, (channels + 255) / 256);
         conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);

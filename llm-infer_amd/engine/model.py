@@ -67,6 +67,10 @@ class DecoderModel(Part):
         self._unit, n = {}, 0
         self._asks = [[len(cache_specs_of(m)) for m in mixers] for mixers in self.layer_mixers]
         self._multi = [[hasattr(m, "cache_specs") for m in mixers] for mixers in self.layer_mixers]
+        # a mixer that reads another run's cache may still keep some of what it asks for to itself (the history of a
+        # convolution on its own queries beside keys and values that it shares): ``keeps_when_reading``, indices
+        # into its ``cache_specs()``
+        self._keeps = [[tuple(getattr(m, "keeps_when_reading", ())) for m in mixers] for mixers in self.layer_mixers]
         for i, e in enumerate(self.schedule):
             if e.cache_from is not None and self._asks[e.layer] != self._asks[self.schedule[e.cache_from].layer]:
                 raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache_from}, whose layer has "
@@ -74,6 +78,12 @@ class DecoderModel(Part):
             for k, count in enumerate(self._asks[e.layer]):
                 self._unit[i, k] = list(range(n, n + count))
                 n += count
+        # the unit behind each thing that each mixer of each run sees: its own, or the one of the run it reads
+        self._seen = {}
+        for i, e in enumerate(self.schedule):
+            for k, count in enumerate(self._asks[e.layer]):
+                self._seen[i, k] = [self._unit[i, k][j] if e.cache_from is None or j in self._keeps[e.layer][k]
+                                    else self._unit[e.cache_from, k][j] for j in range(count)]
         # an embedding may keep state of every sequence too (the token before, say): its units come last
         self._embedding_units = list(range(n, n + len(self._embedding_specs())))
         self._table = collect_params(self)
@@ -141,8 +151,9 @@ class DecoderModel(Part):
     def cache_specs(self) -> list:
         """For each unit (each mixer of each schedule entry, in order, then whatever the embedding keeps of every
         sequence) what it asks of the cache (None: it reads another's)."""
-        return [None if e.cache_from is not None else spec
-                for e in self.schedule for m in self.layer_mixers[e.layer] for spec in cache_specs_of(m)] + self._embedding_specs()
+        return [None if e.cache_from is not None and j not in getattr(m, "keeps_when_reading", ()) else spec
+                for e in self.schedule for m in self.layer_mixers[e.layer]
+                for j, spec in enumerate(cache_specs_of(m))] + self._embedding_specs()
 
     # -- the forward pass of one step ---------------------------------------
     def forward(self, ctx, cache) -> torch.Tensor:
@@ -164,9 +175,8 @@ class DecoderModel(Part):
                 x = self.stream_parts[self._before[i]].forward(x, x0, ctx)       # a new tensor: x0 stays as it is
             elif x is x0 and self.stream_parts and history is None:
                 x = ops.copy_rows(x0)            # the layers add in place, and a later part reads the embedding's output
-            owner = i if e.cache_from is None else e.cache_from
             # one view for a mixer, or the list of its views for one that asks several things of the cache
-            views = [[cache.view(u) for u in self._unit[owner, k]] if multi else cache.view(self._unit[owner, k][0])
+            views = [[cache.view(u) for u in self._seen[i, k]] if multi else cache.view(self._seen[i, k][0])
                      for k, multi in enumerate(self._multi[e.layer])]
             layer = self.layers[e.layer]
             if getattr(layer, "takes_next_norm", False):

@@ -191,14 +191,16 @@ def mixers_library(force=False):
     return _load("libli_mixers.so", MIXER_SOURCES, (), force)
 
 
-HYBRID_SOURCES = ("hybrid.hip", "latent.hip")
+HYBRID_SOURCES = ("hybrid.hip", "latent.hip", "gated.hip")
 
 
 def hybrid_library(force=False):
     """The kernels of hybrid decoders (csrc/hybrid.hip: differential attention over blocks of positions, the
     state-space recurrence and its convolution, the experts' router; csrc/latent.hip: latent attention's
     preparation and products per head, the matrix-memory recurrence, the bigram embedding, the depth-weighted
-    average of the residual stream): a library of its own, as the mixers' is."""
+    average of the residual stream; csrc/gated.hip: the norm of a sub-layer's output with the residual sum, the rotation
+    of half-paired dimensions with the cache write, the clamped gated activation, experts by table): a library of its own,
+    as the mixers' is."""
     return _load("libli_hybrid.so", HYBRID_SOURCES, (), force)
 
 

@@ -1253,7 +1253,7 @@ def diff_tiles(ctx, block=None, window=None):
 
 
 def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale, block, window, lam, out_eps, out_scale,
-                   out_dtype, tiles=None, sink=None, key_shares: int = 1) -> torch.Tensor:
+                   out_dtype, tiles=None, sink=None, key_shares: int = 1, slopes=None, gate=None, gate_col: int = 0) -> torch.Tensor:
     """Attention of ``maps`` softmax maps (1 or 2) over the same values: o = a_1 - lam a_2, then (``out_eps`` not
     None) o divided by its root mean square over dv, times ``out_scale``.  A token at position p sees the keys
     from p - p % block on (``block`` 0: from 0; ``window`` w: at most the last w).  q [T, H, maps * DP] as
@@ -1262,9 +1262,15 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
     ``tiles`` from ``diff_tiles`` for the same block and window (None: every token an item of its own).
     ``sink`` (float32 [H]): every map's sum of weights also counts exp(sink[head]), which has no key and no value.
     ``key_shares`` (a decode step on the matrix cores with four or more query heads on a key/value head): that many
-    workgroups share a token's keys, and a second kernel adds up their states in order."""
-    _dev(q, pos, tok_slot, sink)
+    workgroups share a token's keys, and a second kernel adds up their states in order.
+    ``slopes`` (float32 [H]): the score of the key at position j loses slopes[head] * (p - j); the sink loses nothing.
+    ``gate`` (float32 rows [T, >= gate_col + H]): head h's output is multiplied by sigmoid(gate[t][gate_col + h])."""
+    _dev(q, pos, tok_slot, sink, slopes, gate)
     _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == n_heads), "sink: float32 [H]")
+    _need(slopes is None or (slopes.dtype == torch.float32 and slopes.numel() == n_heads and slopes.is_contiguous()), "slopes: float32 [H]")
+    _need(gate is None or (gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == q.shape[0] and gate.stride(1) == 1
+                           and 0 <= gate_col and gate_col + n_heads <= gate.shape[1]), "gate: float32 rows with a column for every head")
+    extra = (_ptr(slopes), _ptr(gate), gate.stride(0) if gate is not None else 0, int(gate_col))
     t = q.shape[0]
     dp = padded_map_dim(d)
     _need(maps in (1, 2) and dv <= 512 and n_heads % n_kv_heads == 0, "diff_attention: one or two maps, values up to 512 wide")
@@ -1280,7 +1286,7 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
         # (also a 16-bit cache whose sizes the matrix-core kernel does not take)
         _check(hybrid().li_diff_attn(_ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride),
                                      _ptr(page_table), page_table.shape[1], _ptr(pos), _ptr(tok_slot), t, n_heads, n_kv_heads,
-                                     maps, d, dv, *tail), "diff_attn")
+                                     maps, d, dv, *tail[:-1], *extra, tail[-1]), "diff_attn")
         return out
     tile_t0, tile_n, n_tiles = tiles if tiles is not None else (None, None, t)
     if tiles is not None:
@@ -1294,7 +1300,7 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
     _check(_diffattn_lib(dp, vd).li_diffattn(
         _ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
         page_table.shape[1], _ptr(pos), _ptr(tok_slot), _ptr(tile_t0), _ptr(tile_n), n_tiles, n_heads, n_kv_heads, maps, dv,
-        *tail[:-1], key_shares if part is not None else 1, _ptr(part), tail[-1]), "diffattn")
+        *tail[:-1], key_shares if part is not None else 1, _ptr(part), *extra, tail[-1]), "diffattn")
     return out
 
 
@@ -1712,3 +1718,130 @@ def expert_act(z, weights, n_blocks, ff, tail, kind: str, on_input: bool, out_dt
     _check(hybrid().li_expert_act(_ptr(z), _ptr(weights), wcols, _ptr(idx), -1 if col is None else col, _ptr(out), DT[out_dtype],
                                   rows, n_blocks, ff, tail, ACTIVATIONS[kind], int(bool(on_input)), _stream()), "expert_act")
     return out
+
+
+# ---------------------------------------------------------------------------
+# sub-layers between two norms, softmax attention with a sink, a gate a head and a rotation of half-paired dimensions
+# or a bias by distance, clamped gated feed-forwards, experts by table (csrc/gated.hip, in the hybrid library)
+# ---------------------------------------------------------------------------
+def add_bias(rows, col0: int, bias) -> torch.Tensor:
+    """rows[:, col0 : col0 + len(bias)] += bias, in place (float32 rows)."""
+    _dev(rows, bias)
+    _f32_rows(rows, "add_bias rows")
+    _need(bias.dtype == torch.float32 and bias.dim() == 1 and bias.is_contiguous() and 0 <= col0 and col0 + bias.numel() <= rows.shape[1],
+          "add_bias: a float32 vector within the rows")
+    _drop_row_stats(rows)
+    _check(hybrid().li_add_bias(_ptr(rows), rows.shape[1], col0, _ptr(bias), rows.shape[0], bias.numel(), _stream()), "add_bias")
+    return rows
+
+
+def scale_values(x: torch.Tensor, s: float) -> torch.Tensor:
+    """x <- x * s in place (float32, contiguous)."""
+    _dev(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "scale_values: contiguous float32 values")
+    _check(hybrid().li_scale_values(_ptr(x), c_int64(x.numel()), c_float(s), _stream()), "scale_values")
+    return x
+
+
+def conv_plain(rows, col0, channels, weight, history, ctx) -> torch.Tensor:
+    """A causal convolution per channel over ``channels`` columns of the float32 ``rows`` from ``col0`` on, alone: weight
+    float32 [channels, taps] (last column: the current token), no bias, no activation; ``history`` float32
+    [slots, taps - 1, channels] holds every sequence's last inputs and is brought up to date.  Returns float32
+    [T, channels]."""
+    _dev(rows, weight, history)
+    _f32_rows(rows, "conv rows")
+    t, taps = rows.shape[0], weight.shape[1]
+    _need(weight.dtype == torch.float32 and weight.shape == (channels, taps) and 1 <= taps <= 16, "conv weight: float32 [channels, taps <= 16]")
+    _need(0 <= col0 and col0 + channels <= rows.shape[1], "conv: columns beyond the rows")
+    _need(history.dtype == torch.float32 and history.dim() == 3 and tuple(history.shape[1:]) == (max(taps - 1, 1), channels),
+          "conv history: float32 [slots, taps - 1, channels]")
+    _i32(ctx.pos, t, "positions")
+    _i32(ctx.tok_slot, t, "slots")
+    seq_slot, qstart, qlen = _seq_arrays(ctx, t)
+    out = torch.empty((t, channels), dtype=torch.float32, device=rows.device)
+    _check(hybrid().li_conv_plain(_ptr(rows), rows.shape[1], col0, _ptr(weight), None, _ptr(history), _ptr(ctx.pos),
+                                  _ptr(ctx.tok_slot), _ptr(seq_slot), _ptr(qstart), _ptr(qlen), _ptr(out), t, ctx.n_seqs, channels,
+                                  taps, _stream()), "conv_plain")
+    return out
+
+
+def rot_store(rows, q_col, k_col, v_col, inv_freq, rot, pos, tok_slot, kv, n_heads, n_kv_store, d, dv, q_dtype=None) -> torch.Tensor:
+    """From float32 rows with a token's q heads [H, d] from column ``q_col``, k heads [G, d] from ``k_col`` and values
+    [G, dv] from ``v_col`` (it may equal ``k_col``: the values are the keys before their rotation): q and k turned by
+    position in their first ``rot`` dimensions, dimension i paired with i + rot / 2, angle pos * inv_freq[i]; k and v
+    into the pages in matrix-operand order (one map of keys, padded to a multiple of 16).  ``n_kv_store`` 0: nothing
+    is stored (``kv`` may be None, ``q_dtype`` says q's type).  Returns q [T, H, DP] in the cache's type."""
+    _dev(rows, inv_freq, pos, tok_slot)
+    _f32_rows(rows, "rot_store rows")
+    t = rows.shape[0]
+    dp = padded_map_dim(d)
+    _need(0 <= rot <= d and rot % 2 == 0, "rot_store: an even number of rotated dimensions within the head")
+    if rot:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() >= rot // 2, "inv_freq: float32 [rot / 2]")
+    _need(q_col >= 0 and q_col + n_heads * d <= rows.shape[1], "rot_store: q columns beyond the rows")
+    _i32(pos, t, "positions")
+    _i32(tok_slot, t, "slots")
+    if n_kv_store:
+        _need(min(k_col, v_col) >= 0 and k_col + n_kv_store * d <= rows.shape[1] and v_col + n_kv_store * dv <= rows.shape[1],
+              "rot_store: k or v columns beyond the rows")
+        k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, n_kv_store, dp, dv)
+        q_dtype, max_pages = k_pages.dtype, page_table.shape[1]
+    else:
+        k_pages = v_pages = page_table = None
+        page_stride = max_pages = 0
+        _need(q_dtype in DT, "rot_store: q's type")
+    q = torch.empty((t, n_heads, dp), dtype=q_dtype, device=rows.device)
+    _check(hybrid().li_rot_store(_ptr(rows), rows.shape[1], q_col, k_col, v_col, _ptr(inv_freq), rot, _ptr(pos), _ptr(tok_slot),
+                                 _ptr(q), _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table), max_pages,
+                                 DT[q_dtype], t, n_heads, n_kv_store, d, dv, _stream()), "rot_store")
+    return q
+
+
+def rmsnorm_add(x, y, weight, eps: float, bias=None) -> torch.Tensor:
+    """x += (y + bias) / sqrt(mean((y + bias)^2) + eps) * weight, row by row, in place (all float32)."""
+    _dev(x, y, weight, bias)
+    _f32_rows(x, "rmsnorm_add x")
+    _f32_rows(y, "rmsnorm_add y")
+    width = x.shape[1]
+    _need(y.shape == x.shape and weight.dtype == torch.float32 and weight.shape == (width,), "rmsnorm_add: rows of one shape, a float32 weight")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (width,)), "rmsnorm_add: a float32 bias")
+    _drop_row_stats(x)
+    _check(hybrid().li_rmsnorm_add(_ptr(x), _ptr(y), _ptr(bias), _ptr(weight), c_float(eps), x.shape[0], width, _stream()),
+           "rmsnorm_add")
+    return x
+
+
+def clamped_glu(z, bias, out_dtype, n_blocks: int, ff: int, tail: int, limit: float, tail_limit: float, alpha: float,
+                shift: float, weights=None) -> torch.Tensor:
+    """The clamped gated activation of float32 sums z [T, 2 F] over interleaved gate and up columns, F = n_blocks * ff +
+    tail: g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + shift); ``bias`` (float32
+    [2 F], interleaved likewise, or None) is added first; the last ``tail`` outputs take ``tail_limit``; ``weights``
+    (float32 [T, n_blocks (+ 1)]): block e of a row times weights[t][e], the tail times the last column."""
+    _dev(z, bias, weights)
+    _f32_rows(z, "clamped_glu sums")
+    f = n_blocks * ff + tail
+    _need(f > 0 and z.shape[1] == 2 * f, "clamped_glu: [T, 2 (blocks * ff + tail)]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (2 * f,)), "clamped_glu: a float32 bias for every column")
+    _need(weights is None or (weights.dtype == torch.float32 and weights.shape == (z.shape[0], n_blocks + int(tail > 0))),
+          "clamped_glu: a weight for every block")
+    out = torch.empty((z.shape[0], f), dtype=out_dtype, device=z.device)
+    _check(hybrid().li_clamped_glu(_ptr(z), _ptr(bias), _ptr(out), DT[out_dtype], z.shape[0], n_blocks, ff, tail, c_float(limit),
+                                   c_float(tail_limit), c_float(alpha), c_float(shift), _ptr(weights), _stream()), "clamped_glu")
+    return out
+
+
+def table_route(token_ids, table, n_experts: int, gate_logits=None, has_gate: int = 0) -> torch.Tensor:
+    """Routing weights of experts that a table assigns: row ``table[token]`` (int32 [vocab, top]) names a token's experts,
+    each of weight 1 / top.  Returns float32 [T, n_experts (+ 1)], 0 where not named; ``has_gate`` 1: the last column is
+    sigmoid(gate_logits[t]) (float32 [T]), 2: it is 1."""
+    _dev(token_ids, table, gate_logits)
+    t = token_ids.shape[0]
+    _i32(token_ids, t, "token ids")
+    _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous() and 1 <= table.shape[1] <= n_experts,
+          "table_route: int32 [vocab, top]")
+    _need(has_gate != 1 or (gate_logits is not None and gate_logits.dtype == torch.float32 and gate_logits.numel() == t
+                            and gate_logits.is_contiguous()), "table_route: a float32 gate logit for every token")
+    w = torch.empty((t, n_experts + int(bool(has_gate))), dtype=torch.float32, device=token_ids.device)
+    _check(hybrid().li_table_route(_ptr(token_ids), _ptr(table), table.shape[1], n_experts, _ptr(gate_logits), int(has_gate),
+                                   _ptr(w), t, _stream()), "table_route")
+    return w

@@ -87,10 +87,7 @@ class PreNormBlock(Block):
             after = self.sublayers[i + 1].norm if i + 1 < len(self.sublayers) else next_norm
             lazy_after = getattr(after, "can_be_lazy", False)
             ops.expect_norm(x, after.weight if lazy_after else None, after.eps if lazy_after else None)
-            if s.role == "mixer":
-                s.part.forward(h, ctx, next(views), x, owns_cache)
-            else:
-                s.part.forward(h, x)
+            _run_part(s, h, ctx, next(views) if s.role == "mixer" else None, x, owns_cache)
 
 
 @register_block("parallel")
@@ -111,10 +108,47 @@ class ParallelBlock(Block):
         normed = [s.norm.forward(x, out_dtype=torch.float32) if getattr(s.part, "reads_float32", False) else s.norm.forward(x)
                   for s in self.sublayers]
         for s, h in zip(self.sublayers, normed):
-            if s.role == "mixer":
-                s.part.forward(h, ctx, next(views), x, owns_cache)
+            _run_part(s, h, ctx, next(views) if s.role == "mixer" else None, x, owns_cache)
+
+
+def _run_part(s, h, ctx, view, out, owns_cache):
+    """A sub-layer's part on its normed rows ``h``, adding into ``out``; a feed-forward that says ``takes_ctx`` is
+    handed the step too (one that chooses its experts by token id, say)."""
+    if s.role == "mixer":
+        s.part.forward(h, ctx, view, out, owns_cache)
+    elif getattr(s.part, "takes_ctx", False):
+        s.part.forward(h, out, ctx)
+    else:
+        s.part.forward(h, out)
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """x <- x + norm_after(part(norm_before(x))) for each sub-layer in turn: every part stands between two norms,
+    one on what it reads and one on what it adds to the residual stream.  The part adds into cleared float32 rows
+    of its own; the second norm and the residual sum are then one pass over those rows (``ops.rmsnorm_add``).  A
+    part that says ``writes_rows`` is handed rows that it overwrites instead (no clearing), and may hand back a
+    bias that the pass adds first (``forward`` returns it)."""
+
+    def __init__(self, sublayers):
+        super().__init__(sublayers)
+        for s in self.sublayers:
+            if s.norm is None or s.post_norm is None or not hasattr(s.post_norm, "weight"):
+                raise ValueError("a sandwich block has one norm before each part and one with a weight after it")
+
+    def forward(self, x, ctx, cache_views, owns_cache=True):
+        views = iter(cache_views)
+        ops.expect_norm(x, None)                 # no product adds into x itself: no norm rides along
+        for s in self.sublayers:
+            h = s.norm.forward(x)
+            view = next(views) if s.role == "mixer" else None
+            if getattr(s.part, "writes_rows", False):
+                y = torch.empty_like(x)
+                bias = s.part.forward_into(h, y, ctx, view, owns_cache)
             else:
-                s.part.forward(h, x)
+                y, bias = torch.zeros_like(x), None
+                _run_part(s, h, ctx, view, y, owns_cache)
+            ops.rmsnorm_add(x, y, s.post_norm.weight, s.post_norm.eps, bias)
 
 
 @register_block("post_norm")

@@ -81,8 +81,9 @@ class LMHead(Part):
     """logits = h W^T in float32 (src/model/model.cpp:93-98).  ``tied``: W is the embedding
     table (the reference has no tied models: it requires output.weight, model.cpp:35-38)."""
 
-    def __init__(self, *, vocab_size, hidden_size, tied, name="weight", softcap=None, prefix, dtype, device):
-        """``softcap`` c: the logits become c * tanh(logits / c)."""
+    def __init__(self, *, vocab_size, hidden_size, tied, name="weight", softcap=None, scale=1.0, prefix, dtype, device):
+        """``softcap`` c: the logits become c * tanh(logits / c).  ``scale``: the logits are multiplied by it (float32)."""
+        self.scale = float(scale)
         self.vocab_size, self.hidden_size, self.tied, self.name = vocab_size, hidden_size, tied, name
         self.softcap = None if softcap is None else float(softcap)
         if self.softcap is not None and not self.softcap > 0:
@@ -106,4 +107,6 @@ class LMHead(Part):
 
     def forward(self, h):
         logits = ops.linear(h, self.weight, out_dtype=torch.float32)
+        if self.scale != 1.0:
+            ops.scale_values(logits, self.scale)
         return logits if self.softcap is None else ops.softcap(logits, self.softcap)

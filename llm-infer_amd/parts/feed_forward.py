@@ -18,24 +18,42 @@ class GatedMLP(Part):
     Gate and up rows are interleaved into one matrix (row 2j = gate_j, row 2j+1 = up_j),
     so that one product yields both and its epilogue applies the activation before
     anything is written; each row's sum is what it would be alone.
+
+    ``activation`` "clamped_swish": with g = min(gate, ``limit``) and u = clamp(up, -limit, limit) the hidden row is
+    g sigmoid(``alpha`` g) (u + ``up_shift``), computed in float32 on the product's sums.  ``bias``: gate, up and down
+    have biases, added in their products.
     """
 
     takes_lazy_norm = True      # the normed input goes to ops.linear as it comes
+    writes_rows = True          # forward_into overwrites the rows it is handed
 
-    def __init__(self, *, hidden_size, intermediate_size, activation="silu", names=None, prefix, dtype, device):
-        """``names``: local tensor names for gate, up and down."""
-        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", **(names or {})}
-        if activation not in ("silu", "gelu"):
-            raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu and gelu are)")
-        self.mode = ops.EPI_SWIGLU if activation == "silu" else ops.EPI_GEGLU
+    def __init__(self, *, hidden_size, intermediate_size, activation="silu", limit=None, alpha=1.702, up_shift=1.0,
+                 bias=False, names=None, prefix, dtype, device):
+        """``names``: local tensor names for gate, up and down (and gate_bias, up_bias, down_bias)."""
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight",
+                      "gate_bias": "gate_proj.bias", "up_bias": "up_proj.bias", "down_bias": "down_proj.bias", **(names or {})}
+        if activation not in ("silu", "gelu", "clamped_swish"):
+            raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu, gelu and clamped_swish are)")
+        self.clamped = activation == "clamped_swish"
+        if self.clamped and not (limit is not None and float(limit) > 0):
+            raise ValueError("gated_mlp: the clamped activation needs a positive limit")
+        if bias and not self.clamped:
+            raise ValueError("gated_mlp: biases are built for the clamped activation")
+        self.mode = ops.EPI_GEGLU if activation == "gelu" else ops.EPI_SWIGLU
+        self.limit, self.alpha, self.up_shift = float(limit or 0.0), float(alpha), float(up_shift)
+        self.bias = bool(bias)
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
         self.prefix, self.dtype, self.device = prefix, dtype, device
-        self.w_gate_up = self.w_down = None
+        self.w_gate_up = self.w_down = self.b_gate_up = self.b_down = None
 
     def params(self):
         f, d = self.intermediate_size, self.hidden_size
         n = self.names
-        return {n["gate"]: ParamSpec((f, d)), n["up"]: ParamSpec((f, d)), n["down"]: ParamSpec((d, f))}
+        out = {n["gate"]: ParamSpec((f, d)), n["up"]: ParamSpec((f, d)), n["down"]: ParamSpec((d, f))}
+        if self.bias:
+            out.update({n["gate_bias"]: ParamSpec((f,), "vector", "small"), n["up_bias"]: ParamSpec((f,), "vector", "small"),
+                        n["down_bias"]: ParamSpec((d,), "vector", "small")})
+        return out
 
     def bind(self, tensors):
         g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
@@ -44,10 +62,27 @@ class GatedMLP(Part):
         gu = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
         self.w_gate_up = ops.prepare_weight(gu)
         self.w_down = ops.prepare_weight(tensors[self.names["down"]])
+        if self.bias:
+            plain = lambda name: tensors[self.names[name]].as_subclass(torch.Tensor).float()
+            self.b_gate_up = torch.stack([plain("gate_bias"), plain("up_bias")], dim=1).reshape(-1).contiguous()   # interleaved as the rows are
+            self.b_down = plain("down_bias").contiguous()
+
+    def _hidden(self, h):
+        if not self.clamped:
+            return ops.linear(h, self.w_gate_up, self.mode, out_dtype=self.dtype)
+        z = ops.linear(h, self.w_gate_up, out_dtype=torch.float32)
+        return ops.clamped_glu(z, self.b_gate_up, self.dtype, 1, self.intermediate_size, 0, self.limit, self.limit, self.alpha,
+                               self.up_shift)
 
     def forward(self, h, residual):
-        t = ops.linear(h, self.w_gate_up, self.mode, out_dtype=self.dtype)
-        ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)
+        ops.linear(self._hidden(h), self.w_down, ops.EPI_ADD, out=residual)
+        if self.b_down is not None:
+            ops.add_bias(residual, 0, self.b_down)
+
+    def forward_into(self, h, out, ctx=None, view=None, owns_cache=True):
+        """The result written over the float32 rows ``out``; returns the bias that is still to be added to them (or None)."""
+        ops.linear(self._hidden(h), self.w_down, out=out)
+        return self.b_down
 
 
 @register_feed_forward("poly_mlp")
@@ -144,13 +179,25 @@ class RoutedExperts(Part):
 
     def __init__(self, *, hidden_size, n_experts, expert_ff, top, n_identity=0, route_scale=1.0, correction=True,
                  shared_ff=0, shared_gate=True, gated=True, activation="silu", scores="softmax", renormalize=True,
-                 weight_on="output", names=None, prefix, dtype, device):
+                 weight_on="output", routing="router", vocab_size=0, limit=None, shared_limit=None, alpha=1.702,
+                 up_shift=1.0, names=None, prefix, dtype, device):
         if not 1 <= top <= n_experts + n_identity:
             raise ValueError(f"routed experts: top {top} of {n_experts + n_identity} outputs")
         if scores not in ("softmax", "sigmoid") or weight_on not in ("output", "input"):
             raise ValueError("routed experts: scores 'softmax' or 'sigmoid', weight_on 'output' or 'input'")
-        if gated and (activation != "silu" or weight_on != "output"):
-            raise ValueError("routed experts: gated experts are built with silu and the weight on their output")
+        if routing not in ("router", "table"):
+            raise ValueError("routed experts: routing 'router' or 'table'")
+        if routing == "table" and (n_identity or correction or vocab_size < 1):
+            raise ValueError("routed experts: a table names experts with matrices for every token id, without corrections")
+        if gated and (activation not in ("silu", "clamped_swish") or weight_on != "output"):
+            raise ValueError("routed experts: gated experts are built with silu or clamped_swish and the weight on their output")
+        self.clamped = bool(gated) and activation == "clamped_swish"
+        if self.clamped and not (limit is not None and float(limit) > 0):
+            raise ValueError("routed experts: the clamped activation needs a positive limit")
+        self.table_routing, self.vocab_size = routing == "table", int(vocab_size)
+        self.takes_ctx = self.table_routing           # the token ids come with the step
+        self.limit, self.alpha, self.up_shift = float(limit or 0.0), float(alpha), float(up_shift)
+        self.shared_limit = self.limit if shared_limit is None else float(shared_limit)
         if not gated and activation not in ops.ACTIVATIONS:
             raise ValueError(f"routed experts: activation {activation!r} is not built ({', '.join(ops.ACTIVATIONS)} are)")
         self.gated, self.activation, self.sigmoid_scores = bool(gated), activation, scores == "sigmoid"
@@ -159,7 +206,7 @@ class RoutedExperts(Part):
         self.n_identity, self.route_scale, self.correction = n_identity, float(route_scale), bool(correction)
         self.shared_ff, self.shared_gate = int(shared_ff or 0), bool(shared_gate) and bool(shared_ff)
         self.names = {"router": "router.weight", "correction": "router.correction", "expert": "e{}.", "shared": "shared.",
-                      "gate": "gate", "up": "up", "down": "down", "shared_gate": "shared.sg", **(names or {})}
+                      "gate": "gate", "up": "up", "down": "down", "shared_gate": "shared.sg", "table": "table", **(names or {})}
         self.prefix, self.dtype, self.device = prefix, dtype, device
         self.w_router = self.w_gate_up = self.w_down = self.bias = None
 
@@ -170,7 +217,10 @@ class RoutedExperts(Part):
 
     def params(self):
         n, d = self.names, self.hidden_size
-        out = {n["router"]: ParamSpec((self.n_experts + self.n_identity, d), "vector", "wide")}
+        if self.table_routing:
+            out = {n["table"]: ParamSpec((self.vocab_size, self.top), "int", f"distinct:{self.n_experts}")}
+        else:
+            out = {n["router"]: ParamSpec((self.n_experts + self.n_identity, d), "vector", "wide")}
         if self.correction:
             out[n["correction"]] = ParamSpec((self.n_experts + self.n_identity,), "vector", "small")
         for p, f in self._experts():
@@ -203,8 +253,10 @@ class RoutedExperts(Part):
                 parts.append((self._rows(self.w_gate_up, at, rows, g_u), ops.prepare_weight(d_.contiguous())))
                 at += rows
             self.per_expert = parts
-        rows = [tensors[n["router"]].float()] + ([tensors[n["shared_gate"]].float().view(1, d)] if self.shared_gate else [])
-        self.w_router = torch.cat(rows, 0).contiguous()                       # float32: the logits are summed in float32
+        rows = ([] if self.table_routing else [tensors[n["router"]].float()]) + \
+            ([tensors[n["shared_gate"]].float().view(1, d)] if self.shared_gate else [])
+        self.w_router = torch.cat(rows, 0).contiguous() if rows else None     # float32: the logits are summed in float32
+        self.table = tensors[n["table"]] if self.table_routing else None
         self.bias = tensors[n["correction"]] if self.correction else None
 
     @staticmethod
@@ -234,6 +286,13 @@ class RoutedExperts(Part):
             t = self._hidden(h, w_up, weights, None, self.n_experts, 1, self.shared_ff, 0)
             ops.linear(t, w_d, ops.EPI_ADD, out=residual)
 
+    def _gated_hidden(self, rows, w_gu, ff, limit):
+        """One gated expert's hidden rows (no routing weight)."""
+        if not self.clamped:
+            return ops.linear(rows, w_gu, ops.EPI_SWIGLU, out_dtype=self.dtype)
+        z = ops.linear(rows, w_gu, out_dtype=torch.float32)
+        return ops.clamped_glu(z, None, self.dtype, 1, ff, 0, limit, limit, self.alpha, self.up_shift)
+
     def _grouped(self, h, residual, weights):
         if not self.gated:
             return self._grouped_plain(h, residual, weights)
@@ -241,24 +300,38 @@ class RoutedExperts(Part):
         for e, n in enumerate(counts):
             if n:
                 w_gu, w_d = self.per_expert[e]
-                t = ops.linear(ops.gather_rows(h, idx[e], n), w_gu, ops.EPI_SWIGLU, out_dtype=self.dtype)
+                t = self._gated_hidden(ops.gather_rows(h, idx[e], n), w_gu, self.expert_ff, self.limit)
                 ops.scatter_add_rows(residual, ops.linear(t, w_d, out_dtype=torch.float32), idx[e], weights, e)
         if self.shared_ff:
             w_gu, w_d = self.per_expert[self.n_experts]
-            t = ops.linear(h, w_gu, ops.EPI_SWIGLU, out_dtype=self.dtype)
+            t = self._gated_hidden(h, w_gu, self.shared_ff, self.shared_limit)
             ops.scatter_add_rows(residual, ops.linear(t, w_d, out_dtype=torch.float32), None, weights, self.n_experts)
 
-    def forward(self, h, residual):
+    def _weights(self, h, residual, ctx):
+        """The dense row of routing weights of every token (the shared expert's in the last column)."""
+        has_gate = (1 if self.shared_gate else 2) if self.shared_ff else 0
+        if self.table_routing:
+            if ctx is None:
+                raise ValueError("routed experts: a table chooses by token id and needs the step")
+            gate = ops.small_logits(h, self.w_router) if self.shared_gate else None
+            return ops.table_route(ctx.token_ids, self.table, self.n_experts, gate, has_gate)
         logits = ops.small_logits(h, self.w_router)
-        weights = ops.moe_route(logits, self.bias, h, residual, self.n_experts + self.n_identity, self.n_experts, self.top,
-                                (1 if self.shared_gate else 2) if self.shared_ff else 0, self.route_scale,
-                                self.sigmoid_scores, self.renormalize)
+        return ops.moe_route(logits, self.bias, h, residual, self.n_experts + self.n_identity, self.n_experts, self.top,
+                             has_gate, self.route_scale, self.sigmoid_scores, self.renormalize)
+
+    def forward(self, h, residual, ctx=None):
+        weights = self._weights(h, residual, ctx)
         if (self.per_expert is not None and self.n_experts and h.shape[0] * self.top >= self.GROUPED_FROM * self.n_experts
                 and not torch.cuda.is_current_stream_capturing()):
             return self._grouped(h, residual, weights)
         if not self.gated:
             t = self._hidden(h, self.w_gate_up, weights, None, None, self.n_experts, self.expert_ff, self.shared_ff)
             return ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)
-        t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)
-        ops.scale_blocks(t, weights, self.n_experts, self.expert_ff, self.shared_ff)
+        if self.clamped:
+            z = ops.linear(h, self.w_gate_up, out_dtype=torch.float32)
+            t = ops.clamped_glu(z, None, self.dtype, self.n_experts, self.expert_ff, self.shared_ff, self.limit, self.shared_limit,
+                                self.alpha, self.up_shift, weights)
+        else:
+            t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)
+            ops.scale_blocks(t, weights, self.n_experts, self.expert_ff, self.shared_ff)
         ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)

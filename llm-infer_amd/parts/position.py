@@ -13,7 +13,11 @@ class RotaryPosition(Part):
     that starts at dimension i (include/kernels_cpu.hpp:82-100).  ``pairing`` "adjacent"
     rotates (i, i+1) as the reference does; "half" rotates (i/2, i/2 + rotary_dim/2), the order of
     a checkpoint whose q and k rows were never permuted for the reference (docs/gguf.md:487-493).
-    ``scaling_factor`` divides every frequency (linear scaling of positions).
+    ``scaling_factor`` divides every frequency (linear scaling of positions).  ``wavelength_scaling`` {"factor", "low",
+    "high", "original"} stretches by wavelength instead: with l = 2 pi / f, a frequency whose l is shorter than
+    original / high stays, one whose l is longer than original / low becomes f / factor, and between the two
+    s = (original / l - low) / (high - low) blends them, (1 - s) f / factor + s f; the frequencies are then made in
+    float64 and rounded once.
 
     The kernels rotate adjacent pairs only.  A half-paired model runs on them unchanged because a
     score is a sum over the dimensions of a head and does not care about their order: the mixer asks
@@ -31,13 +35,15 @@ class RotaryPosition(Part):
     """
 
     def __init__(self, *, theta: float, rotary_dim: int, head_dim: int, pairing: str = "adjacent",
-                 scaling_factor: float = 1.0, prefix: str = "", dtype, device):
+                 scaling_factor: float = 1.0, wavelength_scaling: dict | None = None, prefix: str = "", dtype, device):
         self.rotary_dim, self.head_dim, self.pairing, self.theta = rotary_dim, head_dim, pairing, float(theta)
         self.scaling_factor = float(scaling_factor)
         self.prefix = prefix
         i = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
         # 1 / powf(theta, i / rotary_dim) in float32, as kernels_cpu.hpp:87
         inv = 1.0 / torch.pow(torch.tensor(float(theta), dtype=torch.float32), i / float(rotary_dim))
+        if wavelength_scaling is not None:
+            inv = scaled_by_wavelength(float(theta), rotary_dim, wavelength_scaling)
         if self.scaling_factor != 1.0:
             # linear scaling: every frequency divided by the factor, i.e. positions counted in its units
             inv = inv / self.scaling_factor
@@ -87,6 +93,26 @@ class RotaryPosition(Part):
         return ctx.shared(wanted[0], lambda: ops.rope_table(self.inv_freq, ctx.pos, ctx.n_tokens))
 
 
+def scaled_by_wavelength(theta: float, rotary_dim: int, scaling: dict) -> torch.Tensor:
+    """theta^(-2i / rotary_dim) for every pair i, stretched by wavelength (see ``RotaryPosition``); float64 throughout,
+    rounded to float32 at the end."""
+    import math
+    factor, low, high, original = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+    if not (factor > 0 and high > low >= 0 and original > 0):
+        raise ValueError("wavelength scaling: factor and original positive, high above low")
+    out = []
+    for i in range(rotary_dim // 2):
+        f = theta ** (-2.0 * i / rotary_dim)
+        wavelength = 2.0 * math.pi / f
+        if wavelength > original / low if low > 0 else False:
+            f = f / factor
+        elif wavelength >= original / high:
+            s = (original / wavelength - low) / (high - low)
+            f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float64).to(torch.float32)
+
+
 def _project(part, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, inv_freq, rotary_dim, fusable, table=None):
     if fusable and part.dtype != torch.float32 and h.dtype == part.dtype:
         k = v = ptab = stride = None
@@ -96,6 +122,22 @@ def _project(part, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, inv_freq, 
                                      n_heads, n_kv_heads, head_dim, part.dtype, cos_sin=table)
     qkv = ops.linear(h, w, out_dtype=torch.float32)
     return part.rotate_store(qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim)
+
+
+@register_position("rope_half")
+class HalfRotaryPosition(RotaryPosition):
+    """The same frequencies for mixers whose own kernel turns dimension i together with i + rotary_dim / 2
+    (``ops.rot_store``): nothing is asked of the mixer's rows, and no table of angles of the step."""
+
+    def __init__(self, **kw):
+        kw.pop("pairing", None)
+        super().__init__(pairing="half", **kw)
+
+    def head_row_order(self, head_dim: int):
+        return None
+
+    def step_table(self):
+        return None
 
 
 @register_position("none")

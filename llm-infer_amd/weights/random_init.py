@@ -3,7 +3,7 @@
 Matrices and tables are N(0, 0.02), norm vectors 1 + N(0, 0.01); a vector whose ``init`` is "small" is
 N(0, 0.02) (a bias), one whose ``init`` is "half" 0.5 + N(0, 0.1) within [0, 1] (mixing weights), one whose ``init``
 is "wide" N(0, 0.4) (a short convolution), one whose ``init`` is "mean" (1 + N(0, 0.2)) / its length (the weights of
-an average).  Every tensor
+an average); an integer table whose ``init`` is "distinct:n" holds in every row different numbers below n.  Every tensor
 has a generator of its own, seeded by (seed, tensor name), so a tensor's values
 depend on neither the order nor the presence of the others.  The reference has
 no such mode.
@@ -30,7 +30,12 @@ def _seed_for(seed: int, name: str) -> int:
 def random_tensor(name: str, spec, seed: int, matrix_dtype: torch.dtype, device="cpu") -> torch.Tensor:
     g = torch.Generator(device=device).manual_seed(_seed_for(seed, name))
     if spec.kind == "int":
-        raise ValueError(f"{name}: integer tables have no random initialisation")
+        if not spec.init.startswith("distinct:"):
+            raise ValueError(f"{name}: integer tables have no random initialisation")
+        # every row names spec.shape[-1] different numbers below n (the experts that a table gives a token id)
+        n = int(spec.init.split(":")[1])
+        order = torch.rand(tuple(spec.shape[:-1]) + (n,), generator=g, device=device).argsort(dim=-1)
+        return order[..., :spec.shape[-1]].to(torch.int32).contiguous()
     if spec.init == "small":         # a bias or another vector around zero
         return MATRIX_STD * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
     if spec.init == "wide":          # weights of a short convolution and the like: of the order of one half
