@@ -1,9 +1,9 @@
 // Kernels of decoders whose sub-layers stand between two norms and whose softmax attention carries a sink, a gate
 // per head and either a rotation of half-paired dimensions or a bias by distance: a bias added to the columns of a
 // product's float32 rows, the rotation of q and k with the write of keys and values into the paged cache, the norm
-// of a sub-layer's output added into the residual stream, the clamped gated activation of a feed-forward (with a
-// bias and with the experts' routing weights), and the routing weights of experts that a table assigns to token ids.
-// The attention itself is hybrid.hip's (float32) and diff_attention.hip's (matrix cores).  Every size is a run-time
+// of a sub-layer's output added into the residual stream, and the routing weights of experts that a table assigns
+// to token ids.  The attention itself is hybrid.hip's (float32) and diff_attention.hip's (matrix cores); the clamped
+// gated activation of the feed-forwards and the biases of products are epilogues of the matrix products (gemm_common.h).  Every size is a run-time
 // value; norms, angles and the residual sum are float32 whatever the type of the matrices.
 #include "common.h"
 
@@ -171,54 +171,6 @@ extern "C" int li_rmsnorm_add(float* x, const float* y, const float* b, const fl
     if (n_rows <= 0) return LI_OK;
     if (width <= 0 || !x || !y || !w) return LI_BAD_ARG;
     rmsnorm_add_kernel<<<n_rows, RA_THREADS, 0, stream>>>(x, y, b, w, eps, width);
-    LI_CHECK_LAUNCH();
-    return LI_OK;
-}
-
-// ---------------------------------------------------------------------------
-// The clamped gated activation on the float32 sums of a product over interleaved rows (column 2j: gate j, column
-// 2j + 1: up j), z [T, 2 F] with F = n_blocks * ff + tail:
-//   g = min(gate + b_gate, limit),  u = clamp(up + b_up, -limit, limit),  out[t][j] = g sigmoid(alpha g) (u + shift)
-// `bias` (float32 [2 F], interleaved as z is) may be null.  The last `tail` outputs take tail_limit.  `weights` not
-// null (float32 [T, n_blocks (+ 1 with a tail)]): block e of a row (an expert's hidden row) is multiplied by
-// weights[t][e], the tail by weights[t][n_blocks]; a weight of 0 writes 0 whatever the sums hold.
-// ---------------------------------------------------------------------------
-__device__ __forceinline__ float clamped_glu_(float g, float u, float limit, float alpha, float shift) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    return g / (1.f + expf(-alpha * g)) * (u + shift);
-}
-
-template <class T>
-__global__ void clamped_glu_kernel(const float* __restrict__ z, const float* __restrict__ bias, T* __restrict__ out,
-                                   int n_blocks, int ff, int tail, float limit, float tail_limit, float alpha, float shift,
-                                   const float* __restrict__ weights) {
-    const int64_t row = blockIdx.x;
-    const int F = n_blocks * ff + tail, wcols = n_blocks + (tail ? 1 : 0);
-    const float* zr = z + row * 2 * F;
-    for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < F; j += gridDim.y * blockDim.x) {
-        const bool in_tail = j >= n_blocks * ff;
-        float w = 1.f;
-        if (weights) w = weights[row * wcols + (in_tail ? n_blocks : j / ff)];
-        float o = 0.f;
-        if (w != 0.f) {
-            const f32x2 gu = *(const f32x2*)(zr + 2 * j);
-            const float g = gu[0] + (bias ? bias[2 * j] : 0.f), u = gu[1] + (bias ? bias[2 * j + 1] : 0.f);
-            o = clamped_glu_(g, u, in_tail ? tail_limit : limit, alpha, shift) * w;
-        }
-        out[row * F + j] = from_f32<T>(o);
-    }
-}
-
-extern "C" int li_clamped_glu(const float* z, const float* bias, void* out, int dt, int n_rows, int n_blocks, int ff, int tail,
-                              float limit, float tail_limit, float alpha, float shift, const float* weights,
-                              hipStream_t stream) {
-    if (n_rows <= 0) return LI_OK;
-    if (n_blocks < 0 || ff < 0 || tail < 0 || n_blocks * ff + tail <= 0) return LI_BAD_ARG;
-    const int F = n_blocks * ff + tail;
-    dim3 grid(n_rows, n_rows >= 1024 ? 1 : (F + 1023) / 1024);
-    DISPATCH_T(dt, (clamped_glu_kernel<T><<<grid, 256, 0, stream>>>(z, bias, (T*)out, n_blocks, ff, tail, limit, tail_limit, alpha,
-                                                                shift, weights)));
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

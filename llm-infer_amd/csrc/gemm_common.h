@@ -3,7 +3,23 @@
 #pragma once
 #include "common.h"
 
-enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3, EPI_GEGLU = 4 };
+enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3, EPI_GEGLU = 4, EPI_BIAS = 5, EPI_CLAMPGLU = 6 };
+
+// What EPI_BIAS and EPI_CLAMPGLU need (handed over where EPI_ROPE's RopeStore is).  EPI_BIAS: C = sums + bias[n].
+// EPI_CLAMPGLU: columns 2j (gate) and 2j + 1 (up), each plus its bias (null: none), give
+//   h[m, j] = g sigmoid(alpha g) (u + shift),  g = min(gate, limit),  u = clamp(up, -limit, limit);
+// the outputs from tail_col on (an expert of another kind behind the others) take tail_limit.
+struct GluParams {
+    const float* bias;          // [N] float32, or null
+    float limit, tail_limit, alpha, shift;
+    int tail_col;               // first output column that takes tail_limit (>= N / 2: none)
+};
+
+__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha, float shift) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-alpha * g)) * (u + shift);
+}
 
 // What the EPI_ROPE epilogue needs: the columns of the product are the q heads, then the k heads,
 // then the v heads of a token; q and k are rotated by the token's position (adjacent pairs), q goes
@@ -27,6 +43,7 @@ struct Epilogue {
     int out_dt;     // DT_* of C (EPI_ADD: always float32)
     int M, N;
     RopeStore rs;
+    GluParams gp;
 };
 
 __device__ __forceinline__ void store_one(void* C, int dt, int64_t i, float v) {
@@ -95,8 +112,29 @@ __device__ __forceinline__ void rope_store4(const RopeStore& r, int m, int head,
     }
 }
 
-// v[0..3] are the results for row m and columns n..n+3 (n a multiple of 4).
-__device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const float* v) {
+// EPI_CLAMPGLU and EPI_BIAS for row m and columns n..n+3 (n a multiple of 4).
+__device__ __forceinline__ void epilogue_extra4(const Epilogue& e, int m, int n, const float* v) {
+    if (m >= e.M || n >= e.N) return;
+    if (e.mode == EPI_CLAMPGLU) {
+        const int64_t row = (int64_t)m * (e.N >> 1);
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+            if (n + j + 1 < e.N) {
+                const int col = (n + j) >> 1;
+                const float g = v[j] + (e.gp.bias ? e.gp.bias[n + j] : 0.f), u = v[j + 1] + (e.gp.bias ? e.gp.bias[n + j + 1] : 0.f);
+                store_one(e.C, e.out_dt, row + col, clamped_glu(g, u, col >= e.gp.tail_col ? e.gp.tail_limit : e.gp.limit,
+                                                                e.gp.alpha, e.gp.shift));
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (n + j < e.N) store_one(e.C, e.out_dt, (int64_t)m * e.N + n + j, v[j] + e.gp.bias[n + j]);
+}
+
+// The other epilogues.  v[0..3] are the results for row m and columns n..n+3 (n a multiple of 4).
+__device__ __forceinline__ void epilogue4_base(const Epilogue& e, int m, int n, const float* v) {
     if (m >= e.M || n >= e.N) return;
     if (e.mode == EPI_ROPE) {
         const RopeStore& r = e.rs;
@@ -159,6 +197,11 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const
     }
 }
 
+// Every epilogue.
+__device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const float* v) {
+    if (e.mode == EPI_CLAMPGLU || e.mode == EPI_BIAS) epilogue_extra4(e, m, n, v);
+    else epilogue4_base(e, m, n, v);
+}
 
 // Sum of the split-K partials in ascending split order, then the epilogue.
 static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int splits, Epilogue e) {
@@ -326,6 +369,14 @@ static void launch_splitk_add_norm(const float* ws, int splits, const Epilogue& 
 static int make_epilogue(Epilogue& e, void* C, int mode, int out_dt, int M, int N, const RopeStore* rs) {
     e.C = C; e.mode = mode; e.out_dt = out_dt; e.M = M; e.N = N;
     e.rs = RopeStore{};
+    e.gp = GluParams{};
+    if (mode == EPI_BIAS || mode == EPI_CLAMPGLU) {
+        const GluParams* gp = (const GluParams*)rs;            // these modes' own parameters come in the same place
+        if (!gp || (mode == EPI_BIAS && !gp->bias) || (mode == EPI_CLAMPGLU && !(gp->limit > 0.f && gp->tail_limit > 0.f)))
+            return LI_BAD_ARG;
+        e.gp = *gp;
+        return LI_OK;
+    }
     if (mode != EPI_ROPE) return LI_OK;
     if (!rs || !rs->pos || !rs->q_out || rs->hd <= 0 || rs->hd % 16 != 0 || rs->H <= 0 || rs->K < 0) return LI_BAD_ARG;
     if (N != (rs->H + 2 * rs->K) * rs->hd || rs->rotary_dim < 0 || rs->rotary_dim > rs->hd || (rs->rotary_dim & 1))
@@ -339,10 +390,10 @@ static int make_epilogue(Epilogue& e, void* C, int mode, int out_dt, int M, int 
 
 static int check_common(const void* X, const void* W, const void* C, int M, int N, int K, int mode, int out_dt) {
     if (!X || !W || (!C && mode != EPI_ROPE) || M < 0 || N <= 0 || K <= 0) return LI_BAD_ARG;
-    if (mode < EPI_STORE || mode > EPI_GEGLU) return LI_BAD_ARG;
+    if (mode < EPI_STORE || mode > EPI_CLAMPGLU) return LI_BAD_ARG;
     if (out_dt < DT_F32 || out_dt > DT_BF16) return LI_BAD_ARG;
     if (mode == EPI_ADD && out_dt != DT_F32) return LI_BAD_ARG;
-    if ((mode == EPI_SWIGLU || mode == EPI_GEGLU) && (N & 1)) return LI_BAD_ARG;
+    if ((mode == EPI_SWIGLU || mode == EPI_GEGLU || mode == EPI_CLAMPGLU) && (N & 1)) return LI_BAD_ARG;
     return LI_OK;
 }
 

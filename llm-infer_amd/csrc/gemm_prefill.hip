@@ -227,6 +227,14 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 // fetch and multiply no rows that are not there).  A: how many steps ahead of their use the loads of W are
 // issued (2; 4 for products of few rows, where one workgroup a CU has to keep enough of W in flight by itself:
 // 8 NI KiB a wave instead of 4 NI; 3 for 65 to 128 rows, where two workgroups may share a CU).
+// The epilogue of one quad: the clamped gated activation and the bias have instantiations of their own, so that the
+// kernel of all the others holds none of their code (and stays within its registers).
+template <int MODE>
+__device__ __forceinline__ void wreg_epilogue(const Epilogue& e, int m, int n, const float* v) {
+    if constexpr (MODE == EPI_CLAMPGLU || MODE == EPI_BIAS) epilogue_extra4(e, m, n, v);
+    else epilogue4_base(e, m, n, v);
+}
+
 template <class T, int NI, int MODE, int MJ = 8, int A = 2>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                         int K, int k_per_split, float* __restrict__ ws, Epilogue e,
@@ -543,8 +551,8 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
                     if (scaled) {
                         const float f = row_ss[256 + min(m, 15)];
                         const float sv[4] = {vv[0] * f, vv[1] * f, vv[2] * f, vv[3] * f};
-                        epilogue4(e, m, col, sv);
-                    } else if (gridDim.z == 1) epilogue4(e, m, col, vv);
+                        wreg_epilogue<MODE>(e, m, col, sv);
+                    } else if (gridDim.z == 1) wreg_epilogue<MODE>(e, m, col, vv);
                     else if (m < e.M) {
                         float* p = ws + ((int64_t)bz * e.M + m) * e.N + col;
 #pragma unroll
@@ -646,7 +654,8 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
     const size_t lds = (stages > strips ? stages : strips) + (size_t)2 * bm * 4 + (256 + 16) * 4;   // and the sums of squares of RowScale
     // the kernels of one epilogue: the residual sum into float32 with whole quads of columns; the
     // rotation with a table of angles
-    const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE : -1;
+    const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE
+                    : (mode == EPI_CLAMPGLU || mode == EPI_BIAS) ? mode : -1;
 #define GO(T, NI, MODE, MJ, A)                                                                            \
     do {                                                                                                  \
         auto kfn = gemm_wreg_kernel<T, NI, MODE, MJ, A>;                                                  \
@@ -663,6 +672,8 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
     do {                                                  \
         if (one == EPI_ADD) GO(T, NI, EPI_ADD, MJ, A);    \
         else if (one == EPI_ROPE) GO(T, NI, EPI_ROPE, MJ, A); \
+        else if (one == EPI_CLAMPGLU) GO(T, NI, EPI_CLAMPGLU, MJ, A); \
+        else if (one == EPI_BIAS) GO(T, NI, EPI_BIAS, MJ, A); \
         else GO(T, NI, -1, MJ, A);                        \
     } while (0)
 #define LAUNCH(T)                                       \

@@ -15,8 +15,8 @@ from ..tensor import Tensor
 
 PAGE = 64
 DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
-EPI_STORE, EPI_ADD, EPI_SWIGLU, EPI_ROPE, EPI_GEGLU = 0, 1, 2, 3, 4
-GATED = (EPI_SWIGLU, EPI_GEGLU)             # gate and up rows interleaved in W, act(gate) * up written
+EPI_STORE, EPI_ADD, EPI_SWIGLU, EPI_ROPE, EPI_GEGLU, EPI_BIAS, EPI_CLAMPGLU = 0, 1, 2, 3, 4, 5, 6
+GATED = (EPI_SWIGLU, EPI_GEGLU, EPI_CLAMPGLU)   # gate and up rows interleaved in W, act(gate) * up written
 _STATUS = {1: "bad argument", 2: "unsupported size or alignment", 3: "HIP launch error"}
 
 
@@ -191,6 +191,24 @@ def lazy_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype):
     return LazyNorm(x, w, eps, out_dtype, xw, ss, scale, row_scales)
 
 
+class _GluParams(ctypes.Structure):
+    _fields_ = [("bias", c_void_p), ("limit", c_float), ("tail_limit", c_float), ("alpha", c_float), ("shift", c_float),
+                ("tail_col", c_int)]
+
+
+def glu_params(bias=None, limit: float = 1.0, tail_limit: float | None = None, alpha: float = 1.702, shift: float = 1.0,
+               tail_col: int | None = None):
+    """What ``linear`` needs for EPI_BIAS (``bias`` float32 [N]) and EPI_CLAMPGLU (gate and up columns interleaved; a bias
+    for every column or None; g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(alpha g) (u + shift); the
+    outputs from ``tail_col`` on take ``tail_limit``).  Keeps the bias alive as long as it lives itself."""
+    _need(bias is None or (bias.dtype == torch.float32 and bias.dim() == 1 and bias.is_contiguous() and bias.is_cuda),
+          "a float32 bias on the device")
+    p = _GluParams(bias.data_ptr() if bias is not None else None, limit, limit if tail_limit is None else tail_limit, alpha, shift,
+                   (1 << 30) if tail_col is None else tail_col)
+    p._bias = bias
+    return p
+
+
 class _NormAfter(ctypes.Structure):
     _fields_ = [("w", c_void_p), ("out", c_void_p), ("out_dt", c_int), ("eps", c_float)]
 
@@ -244,9 +262,11 @@ def _workspace(n_floats: int, device) -> torch.Tensor:
 
 
 def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None = None,
-           out_dtype=None, force: str | None = None, _rope=None) -> torch.Tensor:
+           out_dtype=None, force: str | None = None, _rope=None, params=None) -> torch.Tensor:
     """C = X W^T with the epilogue ``mode``: store, add into ``out`` (float32), or act(gate) * up over
-    interleaved gate/up rows of W (C has N/2 columns; EPI_SWIGLU: silu, EPI_GEGLU: gelu).  ``force`` picks a kernel for tests."""
+    interleaved gate/up rows of W (C has N/2 columns; EPI_SWIGLU: silu, EPI_GEGLU: gelu).  EPI_BIAS stores the sums plus
+    a bias, EPI_CLAMPGLU the clamped gated activation of biased sums; both take ``params`` (``glu_params``).
+    ``force`` picks a kernel for tests."""
     tiled = is_tiled(w)
     wd = w
     w_shape = matrix_shape(w)
@@ -267,6 +287,10 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     if mode == EPI_ADD:
         _need(out is not None and out.dtype == torch.float32, "add epilogue needs a float32 output")
     rs = ctypes.byref(_rope) if _rope is not None else None
+    if mode in (EPI_BIAS, EPI_CLAMPGLU):
+        _need(isinstance(params, _GluParams) and (mode != EPI_BIAS or (params._bias is not None and params._bias.numel() == n)) and
+              (params._bias is None or params._bias.numel() == n), "this epilogue needs its parameters (glu_params), a bias for every column")
+        rs = ctypes.byref(params)
     if mode == EPI_ROPE:
         _need(_rope is not None, "the rotation epilogue needs its arguments (use linear_rope_store)")
     elif out is None:
@@ -1809,25 +1833,6 @@ def rmsnorm_add(x, y, weight, eps: float, bias=None) -> torch.Tensor:
     _check(hybrid().li_rmsnorm_add(_ptr(x), _ptr(y), _ptr(bias), _ptr(weight), c_float(eps), x.shape[0], width, _stream()),
            "rmsnorm_add")
     return x
-
-
-def clamped_glu(z, bias, out_dtype, n_blocks: int, ff: int, tail: int, limit: float, tail_limit: float, alpha: float,
-                shift: float, weights=None) -> torch.Tensor:
-    """The clamped gated activation of float32 sums z [T, 2 F] over interleaved gate and up columns, F = n_blocks * ff +
-    tail: g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + shift); ``bias`` (float32
-    [2 F], interleaved likewise, or None) is added first; the last ``tail`` outputs take ``tail_limit``; ``weights``
-    (float32 [T, n_blocks (+ 1)]): block e of a row times weights[t][e], the tail times the last column."""
-    _dev(z, bias, weights)
-    _f32_rows(z, "clamped_glu sums")
-    f = n_blocks * ff + tail
-    _need(f > 0 and z.shape[1] == 2 * f, "clamped_glu: [T, 2 (blocks * ff + tail)]")
-    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (2 * f,)), "clamped_glu: a float32 bias for every column")
-    _need(weights is None or (weights.dtype == torch.float32 and weights.shape == (z.shape[0], n_blocks + int(tail > 0))),
-          "clamped_glu: a weight for every block")
-    out = torch.empty((z.shape[0], f), dtype=out_dtype, device=z.device)
-    _check(hybrid().li_clamped_glu(_ptr(z), _ptr(bias), _ptr(out), DT[out_dtype], z.shape[0], n_blocks, ff, tail, c_float(limit),
-                                   c_float(tail_limit), c_float(alpha), c_float(shift), _ptr(weights), _stream()), "clamped_glu")
-    return out
 
 
 def table_route(token_ids, table, n_experts: int, gate_logits=None, has_gate: int = 0) -> torch.Tensor:

@@ -66,13 +66,14 @@ class GatedMLP(Part):
             plain = lambda name: tensors[self.names[name]].as_subclass(torch.Tensor).float()
             self.b_gate_up = torch.stack([plain("gate_bias"), plain("up_bias")], dim=1).reshape(-1).contiguous()   # interleaved as the rows are
             self.b_down = plain("down_bias").contiguous()
+        if self.clamped:
+            self.glu = ops.glu_params(self.b_gate_up, self.limit, None, self.alpha, self.up_shift)
 
     def _hidden(self, h):
         if not self.clamped:
             return ops.linear(h, self.w_gate_up, self.mode, out_dtype=self.dtype)
-        z = ops.linear(h, self.w_gate_up, out_dtype=torch.float32)
-        return ops.clamped_glu(z, self.b_gate_up, self.dtype, 1, self.intermediate_size, 0, self.limit, self.limit, self.alpha,
-                               self.up_shift)
+        # biases, clamps and the activation on the product's float32 sums, in its epilogue
+        return ops.linear(h, self.w_gate_up, ops.EPI_CLAMPGLU, out_dtype=self.dtype, params=self.glu)
 
     def forward(self, h, residual):
         ops.linear(self._hidden(h), self.w_down, ops.EPI_ADD, out=residual)
@@ -290,8 +291,8 @@ class RoutedExperts(Part):
         """One gated expert's hidden rows (no routing weight)."""
         if not self.clamped:
             return ops.linear(rows, w_gu, ops.EPI_SWIGLU, out_dtype=self.dtype)
-        z = ops.linear(rows, w_gu, out_dtype=torch.float32)
-        return ops.clamped_glu(z, None, self.dtype, 1, ff, 0, limit, limit, self.alpha, self.up_shift)
+        return ops.linear(rows, w_gu, ops.EPI_CLAMPGLU, out_dtype=self.dtype,
+                          params=ops.glu_params(None, limit, None, self.alpha, self.up_shift))
 
     def _grouped(self, h, residual, weights):
         if not self.gated:
@@ -328,10 +329,11 @@ class RoutedExperts(Part):
             t = self._hidden(h, self.w_gate_up, weights, None, None, self.n_experts, self.expert_ff, self.shared_ff)
             return ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)
         if self.clamped:
-            z = ops.linear(h, self.w_gate_up, out_dtype=torch.float32)
-            t = ops.clamped_glu(z, None, self.dtype, self.n_experts, self.expert_ff, self.shared_ff, self.limit, self.shared_limit,
-                                self.alpha, self.up_shift, weights)
+            # the shared expert's outputs, behind the others', take its own limit
+            t = ops.linear(h, self.w_gate_up, ops.EPI_CLAMPGLU, out_dtype=self.dtype,
+                           params=ops.glu_params(None, self.limit, self.shared_limit, self.alpha, self.up_shift,
+                                                 self.n_experts * self.expert_ff))
         else:
             t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)
-            ops.scale_blocks(t, weights, self.n_experts, self.expert_ff, self.shared_ff)
+        ops.scale_blocks(t, weights, self.n_experts, self.expert_ff, self.shared_ff)
         ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)

@@ -115,7 +115,10 @@ class GatedAttention(Part):
         self.w_in = ops.prepare_weight(torch.cat(rows, 0).contiguous())
         self.wo = ops.prepare_weight(tensors[n["o"]])
         if self.bias:
-            self.b_in = torch.cat([plain(tensors[n[k + "_bias"]]).float() for k in keys]).contiguous()
+            # a bias for every column of the one input product: those of q, k and v, none for the gate's
+            b = torch.cat([plain(tensors[n[k + "_bias"]]).float() for k in keys])
+            pad = torch.zeros(self.n_heads if self.gate else 0, dtype=torch.float32, device=b.device)
+            self.b_in = ops.glu_params(torch.cat([b, pad]).contiguous())
         if self.conv_taps:
             self.conv = torch.cat([plain(tensors[n[k + "_conv"]]).float() for k in keys], 0).contiguous()
         self.sinks = tensors[n["sink"]] if self.sink else None
@@ -146,9 +149,10 @@ class GatedAttention(Part):
             raise ValueError("gated attention: a layer without key and value tensors reads another run's cache, and only such a layer")
         H, G, d, dv = self.n_heads, self.n_kv_heads, self.head_dim, self.v_head_dim
         kv = views[-1].as_tuple()
-        proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         if self.bias:
-            ops.add_bias(proj, 0, self.b_in)
+            proj = ops.linear(h, self.w_in, ops.EPI_BIAS, out_dtype=torch.float32, params=self.b_in)
+        else:
+            proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         rows = ops.conv_plain(proj, 0, self.channels, self.conv, views[0].state, ctx) if self.conv_taps else proj
         q = ops.rot_store(rows, self.q_col, self.k_col, self.v_col, getattr(self.position, "inv_freq", None) if self.rot else None,
                           self.rot, ctx.pos, ctx.tok_slot, kv, H, 0 if self.reads_kv else G, d, dv, kv[0].dtype)

@@ -1,5 +1,8 @@
 """A plain implementation of the Favizen decoder: whole sequences, no cache, one function per mechanism, torch on
 the CPU in the precision of the tensors it is given (float32 or float64).  It shares no code with the engine.
+``round_to`` (a 16-bit type) rounds the activations where a 16-bit engine stores them (the normed rows that enter a
+product, q, k and v as they go to the attention, the heads' outputs, a feed-forward's hidden row) and nothing else: the
+difference to the unrounded run says how much of a 16-bit engine's error is that rounding alone.
 
 Notation: x is the residual stream [T, width]; N(v) = v / sqrt(mean(v^2) + eps).
 
@@ -19,6 +22,10 @@ from __future__ import annotations
 import math
 
 import torch
+
+
+def rounded(t, round_to):
+    return t if round_to is None else t.to(round_to).to(t.dtype)
 
 
 def rms_norm(x, w, eps):
@@ -108,7 +115,7 @@ def gate_heads(o, h, w_g):
     return o * torch.sigmoid(h @ w_g.T)[:, :, None]
 
 
-def attention_mixer(h, W, m):
+def attention_mixer(h, W, m, round_to=None):
     """The rotary mixer with a sliding window; the values are the keys before their rotation."""
     T = h.shape[0]
     H, G, d = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
@@ -120,26 +127,27 @@ def attention_mixer(h, W, m):
     if rot and int(rot["dims"]) > 0:
         f = rope_frequencies(int(rot["dims"]), float(rot["base"]), rot.get("scaling"))
         q, k = rotate(q, pos, f, int(rot["dims"])), rotate(k, pos, f, int(rot["dims"]))
+    q, k, v = rounded(q, round_to), rounded(k, round_to), rounded(v, round_to)
     o = sink_attention(q, k, v, float(m["scale"]), window_mask(T, int(m["mask"]["size"])), W["sink"])
-    return gate_heads(o, h, W["g"]).reshape(T, -1) @ W["o"].T
+    return rounded(gate_heads(o, h, W["g"]), round_to).reshape(T, -1) @ W["o"].T
 
 
-def attention2_keys_values(h, W, m):
+def attention2_keys_values(h, W, m, round_to=None):
     T = h.shape[0]
     G, d, dv = int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
     k = causal_conv(h @ W["k"].T + W["k.b"], W["k.conv"]).view(T, G, d)
     v = causal_conv(h @ W["v"].T + W["v.b"], W["v.conv"]).view(T, G, dv)
-    return k, v
+    return rounded(k, round_to), rounded(v, round_to)
 
 
-def attention2_mixer(h, W, m, kv=None):
+def attention2_mixer(h, W, m, kv=None, round_to=None):
     """The convolved mixer with a distance bias over chunks of positions; ``kv``: another layer's keys and values."""
     T = h.shape[0]
     H, d = int(m["heads"]), int(m["dim"])
-    q = causal_conv(h @ W["q"].T + W["q.b"], W["q.conv"]).view(T, H, d)
-    k, v = kv if kv is not None else attention2_keys_values(h, W, m)
+    q = rounded(causal_conv(h @ W["q"].T + W["q.b"], W["q.conv"]).view(T, H, d), round_to)
+    k, v = kv if kv is not None else attention2_keys_values(h, W, m, round_to)
     o = sink_attention(q, k, v, float(m["scale"]), chunk_mask(T, int(m["mask"]["size"])), W["sink"], slopes(H, h.dtype))
-    return gate_heads(o, h, W["g"]).reshape(T, -1) @ W["o"].T
+    return rounded(gate_heads(o, h, W["g"]), round_to).reshape(T, -1) @ W["o"].T
 
 
 def clamped_glu(g, u, limit: float):
@@ -148,21 +156,21 @@ def clamped_glu(g, u, limit: float):
     return g * torch.sigmoid(1.702 * g) * (u + 1.0)
 
 
-def gated_ff(h, W, prefix: str, limit: float, biases: bool):
+def gated_ff(h, W, prefix: str, limit: float, biases: bool, round_to=None):
     b = (lambda n: W[prefix + n + ".b"]) if biases else (lambda n: 0.0)
     y = clamped_glu(h @ W[prefix + "gate"].T + b("gate"), h @ W[prefix + "up"].T + b("up"), limit)
-    return y @ W[prefix + "down"].T + b("down")
+    return rounded(y, round_to) @ W[prefix + "down"].T + b("down")
 
 
-def table_experts(h, tokens, W, mlp):
+def table_experts(h, tokens, W, mlp, round_to=None):
     top = int(mlp["router"]["top"])
     chosen = W["table"][tokens].long()                      # [T, top]
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e in chosen[t].tolist():
-            out[t] += gated_ff(h[t:t + 1], W, f"e{e}.", float(mlp["expert"]["limit"]), False)[0] / top
+            out[t] += gated_ff(h[t:t + 1], W, f"e{e}.", float(mlp["expert"]["limit"]), False, round_to)[0] / top
     if mlp.get("shared"):
-        out = out + gated_ff(h, W, "shared.", float(mlp["shared"]["limit"]), False) * torch.sigmoid(h @ W["shared.sg"].T)
+        out = out + gated_ff(h, W, "shared.", float(mlp["shared"]["limit"]), False, round_to) * torch.sigmoid(h @ W["shared.sg"].T)
     return out
 
 
@@ -170,7 +178,7 @@ def sub(W, prefix):
     return {k[len(prefix):]: v for k, v in W.items() if k.startswith(prefix)}
 
 
-def forward(config: dict, W: dict, tokens, layers_out: list | None = None):
+def forward(config: dict, W: dict, tokens, layers_out: list | None = None, round_to=None):
     """Logits [T, vocab] of one sequence.  ``W``: tensor name -> tensor (matrices in the dtype to compute in, the
     experts' table as integers).  ``layers_out``: receives the residual stream after every layer."""
     eps = float(config["norm"]["eps"])
@@ -179,25 +187,26 @@ def forward(config: dict, W: dict, tokens, layers_out: list | None = None):
     kept = {}
     for i, layer in enumerate(config["layers"]):
         L, m = sub(W, f"l{i}."), layer["mixer"]
-        h = rms_norm(x, L["norm1"], eps)
+        h = rounded(rms_norm(x, L["norm1"], eps), round_to)
         mix = sub(L, "mix.")
         if layer["type"] == "attention":
-            y = attention_mixer(h, mix, m)
+            y = attention_mixer(h, mix, m, round_to)
         elif layer["type"] == "attention_2":
             if m.get("kv_from") is not None:
-                y = attention2_mixer(h, mix, m, kept[int(m["kv_from"])])
+                y = attention2_mixer(h, mix, m, kept[int(m["kv_from"])], round_to)
             else:
-                kept[i] = attention2_keys_values(h, mix, m)
-                y = attention2_mixer(h, mix, m, kept[i])
+                kept[i] = attention2_keys_values(h, mix, m, round_to)
+                y = attention2_mixer(h, mix, m, kept[i], round_to)
         else:
             raise ValueError(layer["type"])
         x = x + rms_norm(y, L["norm1b"], eps)
         mlp = layer.get("mlp")
         if mlp is not None:
-            h = rms_norm(x, L["norm2"], eps)
+            h = rounded(rms_norm(x, L["norm2"], eps), round_to)
             f = sub(L, "mlp.")
-            y = gated_ff(h, f, "", float(mlp["limit"]), True) if mlp["kind"] == "dense" else table_experts(h, tokens, f, mlp)
+            y = gated_ff(h, f, "", float(mlp["limit"]), True, round_to) if mlp["kind"] == "dense" else \
+                table_experts(h, tokens, f, mlp, round_to)
             x = x + rms_norm(y, L["norm2b"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())
-    return (rms_norm(x, W["final.norm"], eps) @ W["head"].T) * float(config.get("logit_scale", 1.0))
+    return (rounded(rms_norm(x, W["final.norm"], eps), round_to) @ W["head"].T) * float(config.get("logit_scale", 1.0))
