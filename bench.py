@@ -62,7 +62,7 @@ def main() -> int:
                     help="leave out the long contexts, batch 128 and the generation run that the default run adds to points")
     ap.add_argument("--generate", type=int, default=0,
                     help="also generate for this many 128-token prompts with budgets drawn from 16..512 tokens")
-    ap.add_argument("--compare", default="", choices=["", "manirax", "risonex", "dupolorn"],
+    ap.add_argument("--compare", default="", choices=["", "manirax", "risonex", "dupolorn", "favizen"],
                     help="instead of the default workload: prefill and decode throughput of this design at a few "
                          "layer sizes beside the Llama decoder at equal sizes (random weights, a few layers each)")
     ap.add_argument("--sizes", default="", help="with --compare: the layer sizes to run, comma separated (default: all)")
@@ -180,6 +180,28 @@ def compare_configs(design: str, size: dict, layers: int, context: int) -> dict:
         other = {"architecture": "Dupolorn", "canon": {"taps": 3},
                  "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}, "scale": 1.0}, "layers": stack,
                  "logit_softcap": 30.0, "norm": {"eps": 1e-5}, "vocab": size["vocab"], "width": w, "max_positions": context}
+        return {"llama": llama, design: other}
+    if design == "favizen":
+        # the Llama decoder's heads with a sink and a gate a head: two layers whose values are their keys, turned in half
+        # pairs with stretched frequencies, a sliding window of 1,024 positions; two with biases, convolutions of three
+        # taps on q, k and v, a bias by distance and chunks of 1,024 positions, the second of which reads the first's keys
+        # and values; clamped gated feed-forwards: dense of the Llama decoder's width in the first and third layer, else
+        # eight experts of a quarter of it by table, two a token, beside a shared one
+        rot = {"base": 500000.0, "dims": hd, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+        first = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 1024}, "rot": rot}
+        second = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 1024}, "conv": 3}
+        routed = {"kind": "moe", "expert": {"ff": size["ff"] // 4, "limit": 7.0}, "shared": {"ff": size["ff"] // 4, "limit": 7.0},
+                  "router": {"experts": 8, "top": 2}}
+        dense = {"kind": "dense", "ff": size["ff"], "limit": 7.0}
+        stack = []
+        for i in range(layers):
+            kind = ("attention", "attention", "attention_2", "attention_2")[i % 4]
+            mixer = dict(first if kind == "attention" else second)
+            if i % 4 == 3:
+                mixer["kv_from"] = i - 1
+            stack.append({"type": kind, "mixer": mixer, "mlp": dense if i % 2 == 0 else routed})
+        other = {"architecture": "Favizen", "embedding": {"scale": 1.0}, "layers": stack, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+                 "vocab": size["vocab"], "width": w, "max_positions": context}
         return {"llama": llama, design: other}
     assert design == "manirax"
     # the attention of the same heads beside a linear attention of half as many heads with states of hd x hd

@@ -62,12 +62,17 @@ struct StorePages {
     int max_pages;
 };
 
+#define ROT_MAX_PAIRS 256
+
 template <class T>
 __global__ void rot_store_kernel(const float* __restrict__ rows, int stride, int q_col, int k_col, int v_col,
                                  const float* __restrict__ inv_freq, int rot, const int* __restrict__ pos,
                                  const int* __restrict__ tok_slot, T* __restrict__ q_out, StorePages pg, int H, int G,
                                  int d, int dv) {
+    __shared__ float cs[2 * ROT_MAX_PAIRS];               // cos and sin of the token's angles, one pair of them a pair of dimensions
     const int t = blockIdx.x, p = pos[t], DP = round_up(d, 16), half = rot >> 1;
+    for (int j = threadIdx.x; j < half; j += blockDim.x) sincosf((float)p * inv_freq[j], &cs[2 * j + 1], &cs[2 * j]);
+    if (half) __syncthreads();
     const float* row = rows + (int64_t)t * stride;
     T* kp = nullptr;
     T* vp = nullptr;
@@ -88,9 +93,8 @@ __global__ void rot_store_kernel(const float* __restrict__ rows, int stride, int
                 val = src[i];
                 if (i < rot) {
                     const int j = i < half ? i : i - half;
-                    float sn, cs;
-                    sincosf((float)p * inv_freq[j], &sn, &cs);
-                    val = i < half ? val * cs - src[i + half] * sn : val * cs + src[i - half] * sn;
+                    const float c_ = cs[2 * j], s_ = cs[2 * j + 1];
+                    val = i < half ? val * c_ - src[i + half] * s_ : val * c_ + src[i - half] * s_;
                 }
             }
             if (is_q) q_out[((int64_t)t * H + u) * DP + i] = from_f32<T>(val);
@@ -108,6 +112,7 @@ extern "C" int li_rot_store(const float* rows, int stride, int q_col, int k_col,
                             int d, int dv, hipStream_t stream) {
     if (n <= 0) return LI_OK;
     if (H <= 0 || G_store < 0 || d <= 0 || dv <= 0 || rot < 0 || rot > d || (rot & 1) || (rot && !inv_freq)) return LI_BAD_ARG;
+    if (rot > 2 * ROT_MAX_PAIRS) return LI_UNSUPPORTED;
     if (q_col < 0 || q_col + H * d > stride) return LI_BAD_ARG;
     if (G_store && (k_col < 0 || v_col < 0 || k_col + G_store * d > stride || v_col + G_store * dv > stride)) return LI_BAD_ARG;
     StorePages pg{k_pages, v_pages, page_stride, page_table, max_pages};
@@ -121,19 +126,24 @@ extern "C" int li_rot_store(const float* rows, int stride, int q_col, int k_col,
 
 // ---------------------------------------------------------------------------
 // x[t] += (y[t] + b) / sqrt(mean((y[t] + b)^2) + eps) * w: the norm on a sub-layer's output and the residual sum in
-// one pass over the row (b may be null).  One workgroup a row; the row stays in registers up to 8,192 elements.
+// one pass over the row (b may be null).  `next_w` not null: the norm that reads the finished row next is taken too,
+// next[t] = x[t] / sqrt(mean(x[t]^2) + next_eps) * next_w in type TN, while the row is still in registers.
+// One workgroup a row; the row stays in registers up to 8,192 elements (a multiple of 4), else it is read again.
 // ---------------------------------------------------------------------------
 #define RA_THREADS 256
 #define RA_KEEP 8          // 4 elements x RA_KEEP x RA_THREADS = 8,192 elements kept
 
+template <class TN>
 __global__ __launch_bounds__(RA_THREADS) void rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
                                                                  const float* __restrict__ b, const float* __restrict__ w,
-                                                                 float eps, int width) {
+                                                                 float eps, int width, const float* __restrict__ next_w,
+                                                                 float next_eps, TN* __restrict__ next) {
     __shared__ float scratch[16];
     const int64_t row = blockIdx.x;
     const float* yr = y + row * width;
     float* xr = x + row * width;
-    float ss = 0.f;
+    TN* nr = next + row * width;
+    float ss = 0.f, s2 = 0.f;
     if ((width & 3) == 0 && width <= 4 * RA_KEEP * RA_THREADS) {
         f32x4 keep[RA_KEEP];
         const int quads = width >> 2;
@@ -157,20 +167,41 @@ __global__ __launch_bounds__(RA_THREADS) void rmsnorm_add_kernel(float* __restri
                 o[0] += keep[c][0] * r * ww[0]; o[1] += keep[c][1] * r * ww[1];
                 o[2] += keep[c][2] * r * ww[2]; o[3] += keep[c][3] * r * ww[3];
                 *(f32x4*)(xr + 4 * i) = o;
+                keep[c] = o;
+                s2 += o[0] * o[0] + o[1] * o[1] + o[2] * o[2] + o[3] * o[3];
+            }
+        }
+        if (!next_w) return;
+        const float r2 = 1.f / sqrtf(block_sum(s2, scratch) / (float)width + next_eps);
+#pragma unroll
+        for (int c = 0; c < RA_KEEP; ++c) {
+            const int i = threadIdx.x + c * RA_THREADS;
+            if (i < quads) {
+                const f32x4 ww = *(const f32x4*)(next_w + 4 * i);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) nr[4 * i + k] = from_f32<TN>(keep[c][k] * r2 * ww[k]);
             }
         }
         return;
     }
     for (int i = threadIdx.x; i < width; i += RA_THREADS) { const float v = yr[i] + (b ? b[i] : 0.f); ss += v * v; }
     const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
-    for (int i = threadIdx.x; i < width; i += RA_THREADS) xr[i] += (yr[i] + (b ? b[i] : 0.f)) * r * w[i];
+    for (int i = threadIdx.x; i < width; i += RA_THREADS) {
+        const float o = xr[i] + (yr[i] + (b ? b[i] : 0.f)) * r * w[i];
+        xr[i] = o;
+        s2 += o * o;
+    }
+    if (!next_w) return;
+    const float r2 = 1.f / sqrtf(block_sum(s2, scratch) / (float)width + next_eps);
+    for (int i = threadIdx.x; i < width; i += RA_THREADS) nr[i] = from_f32<TN>(xr[i] * r2 * next_w[i]);   // (this thread's own writes)
 }
 
 extern "C" int li_rmsnorm_add(float* x, const float* y, const float* b, const float* w, float eps, int n_rows, int width,
-                              hipStream_t stream) {
+                              const float* next_w, float next_eps, void* next, int next_dt, hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
-    if (width <= 0 || !x || !y || !w) return LI_BAD_ARG;
-    rmsnorm_add_kernel<<<n_rows, RA_THREADS, 0, stream>>>(x, y, b, w, eps, width);
+    if (width <= 0 || !x || !y || !w || (next_w && !next)) return LI_BAD_ARG;
+    if (!next_w) next_dt = DT_F32;
+    DISPATCH_T(next_dt, (rmsnorm_add_kernel<T><<<n_rows, RA_THREADS, 0, stream>>>(x, y, b, w, eps, width, next_w, next_eps, (T*)next)));
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

@@ -1821,8 +1821,10 @@ def rot_store(rows, q_col, k_col, v_col, inv_freq, rot, pos, tok_slot, kv, n_hea
     return q
 
 
-def rmsnorm_add(x, y, weight, eps: float, bias=None) -> torch.Tensor:
-    """x += (y + bias) / sqrt(mean((y + bias)^2) + eps) * weight, row by row, in place (all float32)."""
+def rmsnorm_add(x, y, weight, eps: float, bias=None, next_norm=None) -> torch.Tensor:
+    """x += (y + bias) / sqrt(mean((y + bias)^2) + eps) * weight, row by row, in place (all float32).  ``next_norm``
+    (weight float32 [width], eps, dtype): the RMS norm that reads the finished rows next is taken in the same pass and
+    left for it (``prepared_rmsnorm`` finds it as long as nothing else writes into ``x``)."""
     _dev(x, y, weight, bias)
     _f32_rows(x, "rmsnorm_add x")
     _f32_rows(y, "rmsnorm_add y")
@@ -1830,8 +1832,17 @@ def rmsnorm_add(x, y, weight, eps: float, bias=None) -> torch.Tensor:
     _need(y.shape == x.shape and weight.dtype == torch.float32 and weight.shape == (width,), "rmsnorm_add: rows of one shape, a float32 weight")
     _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (width,)), "rmsnorm_add: a float32 bias")
     _drop_row_stats(x)
-    _check(hybrid().li_rmsnorm_add(_ptr(x), _ptr(y), _ptr(bias), _ptr(weight), c_float(eps), x.shape[0], width, _stream()),
-           "rmsnorm_add")
+    nw = normed = None
+    n_eps, n_dt = 0.0, torch.float32
+    if next_norm is not None:
+        nw, n_eps, n_dt = next_norm
+        _dev(nw)
+        _need(nw.dtype == torch.float32 and nw.shape == (width,) and n_dt in DT, "rmsnorm_add: the next norm's float32 weight and type")
+        normed = torch.empty(x.shape, dtype=n_dt, device=x.device)
+    _check(hybrid().li_rmsnorm_add(_ptr(x), _ptr(y), _ptr(bias), _ptr(weight), c_float(eps), x.shape[0], width, _ptr(nw),
+                                   c_float(n_eps), _ptr(normed), DT[n_dt], _stream()), "rmsnorm_add")
+    if normed is not None:
+        x._li_normed = (normed, nw, float(n_eps), x._version)
     return x
 
 

@@ -126,9 +126,11 @@ def _run_part(s, h, ctx, view, out, owns_cache):
 class SandwichBlock(Block):
     """x <- x + norm_after(part(norm_before(x))) for each sub-layer in turn: every part stands between two norms,
     one on what it reads and one on what it adds to the residual stream.  The part adds into cleared float32 rows
-    of its own; the second norm and the residual sum are then one pass over those rows (``ops.rmsnorm_add``).  A
+    of its own; the second norm and the residual sum are then one pass over those rows (``ops.rmsnorm_add``), which
+    also takes the norm that reads the finished rows next (the next sub-layer's, or the next layer's first).  A
     part that says ``writes_rows`` is handed rows that it overwrites instead (no clearing), and may hand back a
-    bias that the pass adds first (``forward`` returns it)."""
+    bias that the pass adds first (``forward_into`` returns it)."""
+    takes_next_norm = True          # forward accepts ``next_norm``
 
     def __init__(self, sublayers):
         super().__init__(sublayers)
@@ -136,11 +138,20 @@ class SandwichBlock(Block):
             if s.norm is None or s.post_norm is None or not hasattr(s.post_norm, "weight"):
                 raise ValueError("a sandwich block has one norm before each part and one with a weight after it")
 
-    def forward(self, x, ctx, cache_views, owns_cache=True):
+    @staticmethod
+    def _rides(norm):
+        """(weight, eps, dtype) of a norm that the pass before it can take along, or None."""
+        if norm is None or not getattr(norm, "can_be_lazy", False) or getattr(norm, "weight", None) is None:
+            return None
+        return norm.weight, norm.eps, norm.dtype
+
+    def forward(self, x, ctx, cache_views, owns_cache=True, next_norm=None):
+        """``next_norm``: the norm that reads ``x`` after this layer, if the caller knows it."""
         views = iter(cache_views)
         ops.expect_norm(x, None)                 # no product adds into x itself: no norm rides along
-        for s in self.sublayers:
-            h = s.norm.forward(x)
+        for i, s in enumerate(self.sublayers):
+            h = s.norm.forward(x)                # (found ready where the pass before has taken it)
+            after = self._rides(self.sublayers[i + 1].norm if i + 1 < len(self.sublayers) else next_norm)
             view = next(views) if s.role == "mixer" else None
             if getattr(s.part, "writes_rows", False):
                 y = torch.empty_like(x)
@@ -148,7 +159,7 @@ class SandwichBlock(Block):
             else:
                 y, bias = torch.zeros_like(x), None
                 _run_part(s, h, ctx, view, y, owns_cache)
-            ops.rmsnorm_add(x, y, s.post_norm.weight, s.post_norm.eps, bias)
+            ops.rmsnorm_add(x, y, s.post_norm.weight, s.post_norm.eps, bias, after)
 
 
 @register_block("post_norm")

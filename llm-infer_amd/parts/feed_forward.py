@@ -33,7 +33,7 @@ class GatedMLP(Part):
         self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight",
                       "gate_bias": "gate_proj.bias", "up_bias": "up_proj.bias", "down_bias": "down_proj.bias", **(names or {})}
         if activation not in ("silu", "gelu", "clamped_swish"):
-            raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu, gelu and clamped_swish are)")
+            raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu and gelu are, and clamped_swish with a limit)")
         self.clamped = activation == "clamped_swish"
         if self.clamped and not (limit is not None and float(limit) > 0):
             raise ValueError("gated_mlp: the clamped activation needs a positive limit")

@@ -6,10 +6,12 @@ import os
 import torch
 
 
-def rotary(heads, kv_heads, dim, window, dims=None, base=10000.0, scaling=None, scale=None):
+def rotary(heads, kv_heads, dim, window, dims=None, base=10000.0, scaling=None, scale=None, kv_from=None):
     """The mixer with a rotation, a sliding window and values that are the keys."""
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "mask": {"size": window},
          "scale": dim ** -0.5 if scale is None else scale}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
     dims = dim if dims is None else dims
     if dims:
         m["rot"] = {"base": base, "dims": dims}
@@ -58,12 +60,13 @@ TINY_A = config(96, 131, [
 ], eps=1e-6, scale=2.5, logit_scale=0.25)
 
 # a width that the matrix kernels cannot tile; one head; no rotation at all in one layer; five taps and one tap; a layer
-# that reads keys through another mask than their owner's; every expert chosen; no shared expert
+# that reads keys through another mask than their owner's (of either kind); every expert chosen; no shared expert
 TINY_B = config(72, 97, [
     layer(convolved(1, 1, 8, 40, 7, taps=5), dense(40, limit=3.0)),
     layer(rotary(4, 4, 16, 1000, dims=0), moe(4, 4, 8)),
     layer(convolved(1, 1, 8, 40, 33, taps=1, kv_from=0), moe(9, 3, 16, shared=16)),
     layer(rotary(6, 2, 48, 33, dims=16, base=77.0, scaling=(8.0, 1.0, 4.0, 32)), dense(24)),
+    layer(rotary(6, 2, 48, 90, dims=16, base=77.0, scaling=(8.0, 1.0, 4.0, 32), kv_from=3), None),
 ], eps=1e-4, scale=1.0, logit_scale=3.0)
 
 # sizes of real layers, few of them: eight heads of 64 on two key heads, sixteen heads of 128 on one; windows and chunks

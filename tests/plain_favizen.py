@@ -115,19 +115,27 @@ def gate_heads(o, h, w_g):
     return o * torch.sigmoid(h @ w_g.T)[:, :, None]
 
 
-def attention_mixer(h, W, m, round_to=None):
-    """The rotary mixer with a sliding window; the values are the keys before their rotation."""
+def attention_keys_values(h, W, m, round_to=None):
+    """The rotary mixer's keys (turned) and values (the keys as projected)."""
     T = h.shape[0]
-    H, G, d = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
-    q = (h @ W["q"].T).view(T, H, d)
-    k = (h @ W["k"].T).view(T, G, d)
+    k = (h @ W["k"].T).view(T, int(m["kv_heads"]), int(m["dim"]))
     v = k
-    pos = torch.arange(T)
     rot = m.get("rot")
     if rot and int(rot["dims"]) > 0:
-        f = rope_frequencies(int(rot["dims"]), float(rot["base"]), rot.get("scaling"))
-        q, k = rotate(q, pos, f, int(rot["dims"])), rotate(k, pos, f, int(rot["dims"]))
-    q, k, v = rounded(q, round_to), rounded(k, round_to), rounded(v, round_to)
+        k = rotate(k, torch.arange(T), rope_frequencies(int(rot["dims"]), float(rot["base"]), rot.get("scaling")), int(rot["dims"]))
+    return rounded(k, round_to), rounded(v, round_to)
+
+
+def attention_mixer(h, W, m, round_to=None, kv=None):
+    """The rotary mixer with a sliding window; the values are the keys before their rotation; ``kv``: another layer's."""
+    T = h.shape[0]
+    H, d = int(m["heads"]), int(m["dim"])
+    q = (h @ W["q"].T).view(T, H, d)
+    rot = m.get("rot")
+    if rot and int(rot["dims"]) > 0:
+        q = rotate(q, torch.arange(T), rope_frequencies(int(rot["dims"]), float(rot["base"]), rot.get("scaling")), int(rot["dims"]))
+    k, v = kv if kv is not None else attention_keys_values(h, W, m, round_to)
+    q = rounded(q, round_to)
     o = sink_attention(q, k, v, float(m["scale"]), window_mask(T, int(m["mask"]["size"])), W["sink"])
     return rounded(gate_heads(o, h, W["g"]), round_to).reshape(T, -1) @ W["o"].T
 
@@ -190,7 +198,9 @@ def forward(config: dict, W: dict, tokens, layers_out: list | None = None, round
         h = rounded(rms_norm(x, L["norm1"], eps), round_to)
         mix = sub(L, "mix.")
         if layer["type"] == "attention":
-            y = attention_mixer(h, mix, m, round_to)
+            if m.get("kv_from") is None:
+                kept[i] = attention_keys_values(h, mix, m, round_to)
+            y = attention_mixer(h, mix, m, round_to, kept[i if m.get("kv_from") is None else int(m["kv_from"])])
         elif layer["type"] == "attention_2":
             if m.get("kv_from") is not None:
                 y = attention2_mixer(h, mix, m, kept[int(m["kv_from"])], round_to)

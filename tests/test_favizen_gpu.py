@@ -95,7 +95,18 @@ def test_bias_scale_and_the_norm_with_the_residual_sum(lib):
             z = y.double() + (0 if bias is None else bias.double())
             ref = x.double() + z / torch.sqrt(z.pow(2).mean(-1, keepdim=True) + 1e-3) * w.double()
             got = ops.rmsnorm_add(x.clone().to(DEV), y.to(DEV), w.to(DEV), 1e-3, None if bias is None else bias.to(DEV)).cpu()
-            assert error(got, ref) < 1e-6, width
+            assert error(got, ref) < 3e-6, width
+            # with the norm that reads the finished rows next taken along
+            for dt in (torch.float32, torch.bfloat16):
+                xd, w2 = x.clone().to(DEV), (w * 0.5 + 1).to(DEV)
+                ops.rmsnorm_add(xd, y.to(DEV), w.to(DEV), 1e-3, None if bias is None else bias.to(DEV), (w2, 1e-5, dt))
+                assert error(xd.cpu(), ref) < 3e-6
+                ready = ops.prepared_rmsnorm(xd, w2, 1e-5, dt)
+                assert ready is not None and ops.prepared_rmsnorm(xd, w2, 1e-4, dt) is None
+                nref = ref / torch.sqrt(ref.pow(2).mean(-1, keepdim=True) + 1e-5) * w2.double().cpu()
+                assert error(ready.cpu(), nref) < (3e-6 if dt == torch.float32 else 1e-2)
+                ops.add_bias(xd, 0, w2)                                   # anything written into the rows voids what was prepared
+                assert ops.prepared_rmsnorm(xd, w2, 1e-5, dt) is None
     rows_ = torch.randn(7, 50, generator=g)
     b = torch.randn(20, generator=g)
     got = ops.add_bias(rows_.clone().to(DEV), 13, b.to(DEV)).cpu()
