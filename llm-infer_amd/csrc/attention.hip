@@ -40,6 +40,19 @@ struct CachePtrs {
     int max_pages;
 };
 
+// What a prompt's attention may carry beside the causal mask and the window (all off when zero / null):
+// `block` b: a token at position p reads no key before p - p % b; `sink` [H]: every head's sum of weights also counts
+// exp(sink[h]), a score with no key and no value that is not scaled; `slopes` [H]: the score of the key at position j
+// loses slopes[h] * (p - j); `gate`: head h's output is multiplied by sigmoid(gate[token][gate_col + h]) (float32 rows of
+// gate_stride numbers).
+struct AttnExtras {
+    int block;
+    const float* sink;
+    const float* slopes;
+    const float* gate;
+    int gate_stride, gate_col;
+};
+
 template <class T>
 struct WaveAttn {
     typedef typename Vec<T>::v8 v8;
@@ -270,6 +283,18 @@ struct PrefillWave {
             }
     }
 
+    // Every score loses `per` for every position between this lane's row (at position pos) and its key.
+    __device__ __forceinline__ void bias(f32x16 (&n)[2], int t0, int pos, float per) const {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int t = t0 + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                n[b][r] = fmaf(-per, (float)(pos - t), n[b][r]);
+            }
+    }
+
     // The running maximum takes in a page's largest score mx; alpha is what the sums so far are
     // to be multiplied by before that page is added.
     __device__ __forceinline__ void take_max(float mx, float scale2) {
@@ -324,7 +349,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     const T* __restrict__ q, T* __restrict__ out, CachePtrs c, const int* __restrict__ tile_seq,
     const int* __restrict__ tile_q0, const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
     const int* __restrict__ seq_qlen, const int* __restrict__ seq_ctx, int H, int K, float scale, int window,
-    int GW) {
+    int GW, AttnExtras ex) {
     typedef typename Vec<T>::v8 v8;
     constexpr int KE = PAGE * HD, VE = PAGE * DB * 32;           // elements of a head's keys / values in a page
     constexpr int KL = KE / 512, VL = VE / 512;                  // loads of 1 KiB (a wave's) that bring them
@@ -354,7 +379,15 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     const int64_t tok = seq_qstart[seq] + qi;
     PrefillWave<T> a;
     a.init(live ? q + (tok * H + h) * HD : nullptr);
-    const int lo = (window > 0 && live) ? max(0, pos - window + 1) : 0;
+    // the first key that a token at position p0 reads (never later for an earlier token)
+    auto first_key = [&](int p0) {
+        int f = window > 0 ? max(0, p0 - window + 1) : 0;
+        if (ex.block > 0) f = max(f, p0 - p0 % ex.block);
+        return f;
+    };
+    const int lo = live ? first_key(pos) : 0;
+    // scores are kept unscaled until the exponential: the bias by distance in their units
+    const float per = ex.slopes ? ex.slopes[h] / scale : 0.f;
     int lo_max = lo, hi_min = pos;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -363,9 +396,9 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     }
     lo_max = __builtin_amdgcn_readfirstlane(lo_max);
     hi_min = __builtin_amdgcn_readfirstlane(hi_min);
-    const int p_lo = (window > 0 ? max(0, base + q0 - window + 1) : 0) / PAGE;
+    const int p_lo = first_key(base + q0) / PAGE;
     const int p_hi = (base + min(q0 + TT - 1, qlen - 1)) / PAGE;
-    const int wp_lo = (window > 0 ? max(0, base + first - window + 1) : 0) / PAGE;
+    const int wp_lo = first_key(base + first) / PAGE;
     const int wp_hi = wave_live ? (base + min(first + 31, qlen - 1)) / PAGE : -1;
     const int* table = c.page_table + (int64_t)seq_slot[seq] * c.max_pages;
     const T* kbase = (const T*)c.k + (int64_t)kvh * k_head_elems(HD);
@@ -413,6 +446,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
         for (; p < own_lo - 1; ++p) step(p);
         step(p);                                                 // p = own_lo - 1: the first page's scores
         a.template scores<false>(kaddr(p + 1), sa, sa, pf, scale2);
+        if (per != 0.f) a.bias(sa, (p + 1) * PAGE, pos, per);
         if (is_masked(p + 1)) a.mask(sa, (p + 1) * PAGE, lo, pos);
         {
             float mx = -INFINITY;
@@ -424,6 +458,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
         auto both = [&](f32x16 (&cur)[2], f32x16 (&nxt)[2]) {    // page p from cur, the scores of p+1 into nxt
             step(p);
             a.template scores<true>(kaddr(p + 1), nxt, cur, pf, scale2);
+            if (per != 0.f) a.bias(nxt, (p + 1) * PAGE, pos, per);
             if (is_masked(p + 1)) a.mask(nxt, (p + 1) * PAGE, lo, pos);
             a.rescale();
             a.template mix<true>(vaddr(p), pf, nxt, scale2);
@@ -450,8 +485,15 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     }
     for (; p <= p_hi; ++p) step(p);
     __builtin_amdgcn_s_waitcnt(0x0F70);                          // nothing of this workgroup's is still on its way into LDS
-    const float inv = 1.f / a.total();
+    float inv;
+    if (ex.sink) {
+        // the sink joins the sum as one more weight, exp(sink - maximum), with nothing to add to the output
+        const float s2 = ex.sink[h] * LOG2E, big = fmaxf(a.m, s2);
+        const float f = __builtin_amdgcn_exp2f(a.m - big);        // (0 for a row that saw no key)
+        inv = f / (a.total() * f + __builtin_amdgcn_exp2f(s2 - big));
+    } else inv = 1.f / a.total();
     if (!live) return;
+    if (ex.gate) inv *= 1.f / (1.f + expf(-ex.gate[tok * ex.gate_stride + ex.gate_col + h]));
     T* orow = out + (tok * H + h) * HD;
 #pragma unroll
     for (int b = 0; b < DB; ++b)
@@ -672,10 +714,13 @@ static int check_heads(int H, int K) { return (H > 0 && K > 0 && H % K == 0) ? L
 extern "C" int li_attn_prefill(const void* q, void* out, int dt, const void* k, const void* v, int64_t page_stride,
                                const int* page_table, int max_pages, const int* tile_seq, const int* tile_q0,
                                int n_tiles, const int* seq_slot, const int* seq_qstart, const int* seq_qlen,
-                               const int* seq_ctx, int H, int K, float scale, int window, hipStream_t stream) {
+                               const int* seq_ctx, int H, int K, float scale, int window, int key_block, const float* sink,
+                               const float* slopes, const float* gate, int gate_stride, int gate_col, hipStream_t stream) {
     if (check_heads(H, K)) return LI_BAD_ARG;
+    if (key_block < 0 || !(scale > 0.f) || (gate && (gate_col < 0 || gate_col + H > gate_stride))) return LI_BAD_ARG;
     if (n_tiles <= 0) return LI_OK;
     CachePtrs c{k, v, page_stride, page_table, max_pages};
+    const AttnExtras ex{key_block, sink, slopes, gate, gate_stride, gate_col};
     const int G = H / K;
     const int gw = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);        // query heads of a KV head per workgroup
     dim3 grid(n_tiles * gw, K * (G / gw)), block(256);
@@ -686,7 +731,7 @@ extern "C" int li_attn_prefill(const void* q, void* out, int dt, const void* k, 
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
             return LI_HIP_ERROR;                                                                               \
         kfn<<<grid, block, lds, stream>>>((const T*)q, (T*)out, c, tile_seq, tile_q0, seq_slot, seq_qstart,    \
-                                          seq_qlen, seq_ctx, H, K, scale, window, gw);                         \
+                                          seq_qlen, seq_ctx, H, K, scale, window, gw, ex);                     \
     } while (0)
     if (dt == DT_F16) GO(f16);
     else if (dt == DT_BF16) GO(bf16);

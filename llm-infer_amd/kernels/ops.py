@@ -680,12 +680,20 @@ def prefill_meta(ctx) -> dict:
                 seq_qstart=ctx.seq_qstart, seq_qlen=ctx.seq_qlen, seq_ctx=ctx.seq_ctx)
 
 
-def attention_prefill(q, kv, meta, n_heads, n_kv_heads, head_dim, scale, window) -> torch.Tensor:
+def attention_prefill(q, kv, meta, n_heads, n_kv_heads, head_dim, scale, window, block=None, sink=None, slopes=None,
+                      gate=None, gate_col: int = 0) -> torch.Tensor:
     """16-bit attention for a step with whole prompts.  ``kv``: (k_pages, v_pages, page_stride,
     page_table); ``meta``: dict of int32 device arrays tile_seq, tile_q0, seq_slot, seq_qstart,
-    seq_qlen, seq_ctx and the int n_tiles."""
+    seq_qlen, seq_ctx and the int n_tiles.  ``block`` b: a token at position p reads no key before p - p % b;
+    ``sink`` (float32 [H]): every head's sum of weights also counts exp(sink[h]); ``slopes`` (float32 [H]): the
+    score of the key at position j loses slopes[h] * (p - j); ``gate`` (float32 rows [T, >= gate_col + H]): head
+    h's output is multiplied by sigmoid(gate[t][gate_col + h])."""
     k_pages, v_pages, page_stride, page_table = kv
-    _dev(q, k_pages, v_pages, page_table)
+    _dev(q, k_pages, v_pages, page_table, sink, slopes, gate)
+    for name, vec in (("sink", sink), ("slopes", slopes)):
+        _need(vec is None or (vec.dtype == torch.float32 and vec.numel() == n_heads and vec.is_contiguous()), f"{name}: float32 [H]")
+    _need(gate is None or (gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == q.shape[0] and gate.stride(1) == 1
+                           and 0 <= gate_col and gate_col + n_heads <= gate.shape[1]), "gate: float32 rows with a column for every head")
     _need(q.dtype in (torch.float16, torch.bfloat16) and q.shape[1:] == (n_heads, head_dim), "q: 16-bit [T, H, hd]")
     _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, q.dtype)
     out = torch.empty_like(q)
@@ -693,7 +701,8 @@ def attention_prefill(q, kv, meta, n_heads, n_kv_heads, head_dim, scale, window)
         _ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
         page_table.shape[1], _ptr(meta["tile_seq"]), _ptr(meta["tile_q0"]), meta["n_tiles"], _ptr(meta["seq_slot"]),
         _ptr(meta["seq_qstart"]), _ptr(meta["seq_qlen"]), _ptr(meta["seq_ctx"]), n_heads, n_kv_heads,
-        c_float(scale), int(window or 0), _stream()), "attn_prefill")
+        c_float(scale), int(window or 0), int(block or 0), _ptr(sink), _ptr(slopes), _ptr(gate),
+        gate.stride(0) if gate is not None else 0, int(gate_col), _stream()), "attn_prefill")
     return out
 
 

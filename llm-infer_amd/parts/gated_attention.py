@@ -40,8 +40,11 @@ class GatedAttention(Part):
       a layer whose cache another layer reads with another mask keeps what both need).
 
     The input products are one product against [W_q; W_k; W_v; W_g].  The cache keeps keys (after rotation or
-    convolution) and values in the matrix cores' operand order; a 16-bit model runs prompts and decode steps through
-    the matrix-core kernel of ``diff_attention`` with one map, a float32 model one workgroup per (token, head).
+    convolution) and values in the matrix cores' operand order (one map of keys: the layout that the softmax decoder's
+    kernels read too).  A 16-bit model whose keys and values have one size that is a multiple of 16 runs prompts
+    through the softmax decoder's prompt kernel (``ops.attention_prefill``, which takes the sink, the slopes, the
+    blocks and the gate); every other size, and every decode step, runs through the matrix-core kernel of
+    ``diff_attention`` with one map; a float32 model runs one workgroup per (token, head).
     Scores, weights, angles, the sink and the gate are float32 whatever the matrices' type.  ``names``: local tensor
     names."""
 
@@ -156,6 +159,12 @@ class GatedAttention(Part):
         rows = ops.conv_plain(proj, 0, self.channels, self.conv, views[0].state, ctx) if self.conv_taps else proj
         q = ops.rot_store(rows, self.q_col, self.k_col, self.v_col, getattr(self.position, "inv_freq", None) if self.rot else None,
                           self.rot, ctx.pos, ctx.tok_slot, kv, H, 0 if self.reads_kv else G, d, dv, kv[0].dtype)
+        if self.dtype != torch.float32 and not ctx.is_decode and d == dv and d % 16 == 0 and d <= 256:
+            # prompts of a 16-bit model whose keys and values have one size the kernels take as it is: the softmax
+            # decoder's own prompt kernel (pages through LDS, scores of the next page under the weights of this one)
+            a = ops.attention_prefill(q, kv, ops.prefill_meta(ctx), H, G, d, self.scale, self.window, self.block, self.sinks,
+                                      self.slopes, proj if self.gate else None, self.gate_col)
+            return a.view(a.shape[0], H * dv)
         sixteen = self.dtype != torch.float32 and ops.diff_attention_fits(d, dv)
         return ops.diff_attention(q, kv, ctx.pos, ctx.tok_slot, H, G, 1, d, dv, self.scale, self.block, self.window, 0.0, None, 1.0,
                                   self.dtype, ops.diff_tiles(ctx, self.block, self.window) if sixteen else None, sink=self.sinks,

@@ -104,7 +104,7 @@ def test_bias_scale_and_the_norm_with_the_residual_sum(lib):
                 ready = ops.prepared_rmsnorm(xd, w2, 1e-5, dt)
                 assert ready is not None and ops.prepared_rmsnorm(xd, w2, 1e-4, dt) is None
                 nref = ref / torch.sqrt(ref.pow(2).mean(-1, keepdim=True) + 1e-5) * w2.double().cpu()
-                assert error(ready.cpu(), nref) < (3e-6 if dt == torch.float32 else 1e-2)
+                assert error(ready.cpu(), nref) < (3e-6 if dt == torch.float32 else 3e-2)
                 ops.add_bias(xd, 0, w2)                                   # anything written into the rows voids what was prepared
                 assert ops.prepared_rmsnorm(xd, w2, 1e-5, dt) is None
     rows_ = torch.randn(7, 50, generator=g)
