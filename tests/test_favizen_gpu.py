@@ -21,7 +21,7 @@ import trace_util as TU
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
 TOL = {"float32": 1e-4, "bfloat16": 3e-2}
-SHOWS = {"float32": 20.0, "bfloat16": 3.0}      # a fault shows if it moves the result by this many tolerances
+SHOWS = {"float32": 20.0, "bfloat16": 2.0}      # a fault shows if it moves the result by this many tolerances
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
@@ -252,6 +252,9 @@ SCHEDULES = {
     M.convolved(1, 1, 8, 40, 7, taps=5),                                         # chunks shorter than a tile, five taps
     M.convolved(16, 1, 128, 64, 130, taps=4),                                    # sixteen heads on one key head
     M.convolved(5, 5, 32, 16, 64, taps=1),                                       # one tap, chunk = page
+    M.convolved(8, 2, 64, 64, 70, taps=3),                                       # keys and values of one size: the prompt kernel
+    M.convolved(6, 1, 32, 32, 200, taps=2),                                      # with slopes and chunks, six heads on one key head
+    M.rotary(4, 2, 24, 70, dims=8),                                              # a window on the kernel of padded sizes
 ], ids=lambda m: f"{m[0]}-{m[1]['heads']}x{m[1]['dim']}-{m[1]['mask']['size']}")
 def test_mixer_alone(lib, mixer, dtype, schedule):
     width, n, m_ = 96, 200, 40
@@ -273,8 +276,13 @@ def test_mixer_alone(lib, mixer, dtype, schedule):
 # ---------------------------------------------------------------------------- edges, far keys, sinks
 def edge_case(kind, dtype_w=torch.bfloat16):
     """A one-layer model whose token 7 has a key that stands out, the layer's mask size, and the sizes one off."""
+    # (keys and values of one size that is a multiple of 16 run prompts on one kernel, other sizes on another)
     if kind == "window":
         mixer, size = M.rotary(4, 2, 32, 70, dims=16, base=300.0, scaling=(4.0, 1.0, 2.0, 30)), 70
+    elif kind == "window_padded":
+        mixer, size = M.rotary(4, 2, 24, 70, dims=8, base=300.0), 70
+    elif kind == "chunk":
+        mixer, size = M.convolved(4, 2, 32, 32, 70, taps=1), 70
     else:
         mixer, size = M.convolved(4, 2, 32, 16, 70, taps=1), 70
     cfg = M.config(64, 60, [M.layer(mixer, M.dense(48))], scale=2.0, logit_scale=0.5)
@@ -283,7 +291,7 @@ def edge_case(kind, dtype_w=torch.bfloat16):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("kind", ["window", "chunk"])
+@pytest.mark.parametrize("kind", ["window", "window_padded", "chunk", "chunk_other"])
 def test_a_key_just_inside_and_just_outside_the_mask_in_prompts_portions_and_decoding(lib, kind, dtype, tmp_path):
     cfg, W, size = edge_case(kind)
     Wd = M.widen(W)
@@ -291,16 +299,17 @@ def test_a_key_just_inside_and_just_outside_the_mask_in_prompts_portions_and_dec
     base = [t if t != 7 else 8 for t in tokens(cfg, n, 5)]
     # the token that stands out sits so that the probe rows see it just still, and the next row no more:
     # window: the key at 20 is seen up to position 20 + size - 1; chunk: the key at size - 3 is seen up to size - 1
-    at = 20 if kind == "window" else size - 3
+    window = kind.startswith("window")
+    at = 20 if window else size - 3
     toks = list(base)
     toks[at] = 7
-    last_seen = at + size - 1 if kind == "window" else size - 1
+    last_seen = at + size - 1 if window else size - 1
     ref = P.forward(cfg, Wd, toks)
     tol = M.tolerance(dtype, ref, P.forward(cfg, Wd, toks, round_to=torch.bfloat16))
     # the plain implementation alone: one position more or less of mask moves the rows at the edge far beyond the tolerance
     for wrong in (size - 1, size + 1):
         off = P.forward(M.with_mask(cfg, 0, wrong), Wd, toks)
-        edge_rows = [last_seen, last_seen + 1] if kind == "window" else [last_seen - 1, last_seen, last_seen + 1, last_seen + 2]
+        edge_rows = [last_seen, last_seen + 1] if window else [last_seen - 1, last_seen, last_seen + 1, last_seen + 2]
         assert M.row_error(off[edge_rows], ref[edge_rows]) > SHOWS[dtype] * tol, (kind, wrong)
     eng = load(lib, tmp_path, cfg, W, dtype)
     reqs = {"a": toks}
@@ -311,11 +320,14 @@ def test_a_key_just_inside_and_just_outside_the_mask_in_prompts_portions_and_dec
         assert M.row_error(got, ref) < tol, (kind, name)
 
 
+@pytest.mark.parametrize("vdim", [16, 32])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_far_key_among_hundreds_and_a_sink_that_outweighs_it(lib, dtype, tmp_path):
-    mixer = M.convolved(4, 1, 32, 16, 1000, taps=2)
+def test_a_far_key_among_hundreds_and_a_sink_that_outweighs_it(lib, dtype, vdim, tmp_path):
+    mixer = M.convolved(4, 1, 32, vdim, 1000, taps=2)
     cfg = M.config(64, 60, [M.layer(mixer, None)], scale=2.0)
-    W = M.stand_out(M.random_weights(cfg, 78), cfg, 0, 7, strength=9.0)
+    # (strong enough to outweigh hundreds of keys and, in the heads with small slopes, the bias over 700 positions; not so
+    # strong that no sink could weigh against it)
+    W = M.stand_out(M.random_weights(cfg, 78), cfg, 0, 7, strength=5.0 if vdim == 16 else 3.5)
     n = 700
     base = [t if t != 7 else 8 for t in tokens(cfg, n, 6)]
     toks = list(base)

@@ -39,8 +39,10 @@ def draw(seed):
             else:
                 kp, vp = r.choice(PAIRS)
                 G = r.choice([1, 2, 3])
-                mixer = M.convolved(G * r.choice([1, 2, 4, 8]), G, r.randint(max(1, kp - 15), kp), r.randint(vp - 31, vp), size,
-                                    taps=r.randint(1, 6), scale=r.uniform(0.05, 0.3))
+                d, dv = r.randint(max(1, kp - 15), kp), r.randint(vp - 31, vp)
+                if r.random() < 0.3:
+                    d = dv = r.choice([16, 32, 48, 64])                           # one size, a multiple of 16: the prompt kernel
+                mixer = M.convolved(G * r.choice([1, 2, 4, 8]), G, d, dv, size, taps=r.randint(1, 6), scale=r.uniform(0.05, 0.3))
                 owners.append(i)
         kind = r.random()
         if kind < 0.2:
