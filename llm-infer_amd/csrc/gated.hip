@@ -133,7 +133,9 @@ extern "C" int li_rot_store(const float* rows, int stride, int q_col, int k_col,
 #define RA_THREADS 256
 #define RA_KEEP 8          // 4 elements x RA_KEEP x RA_THREADS = 8,192 elements kept
 
-template <class TN>
+// EARLY (the few rows of a decode step): everything the row needs is asked for at once (y, the bias, x and the weight), so
+// that a row waits for memory once and not once a phase; many rows fill the chip anyway and do better with fewer registers.
+template <class TN, bool EARLY>
 __global__ __launch_bounds__(RA_THREADS) void rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
                                                                  const float* __restrict__ b, const float* __restrict__ w,
                                                                  float eps, int width, const float* __restrict__ next_w,
@@ -145,13 +147,17 @@ __global__ __launch_bounds__(RA_THREADS) void rmsnorm_add_kernel(float* __restri
     TN* nr = next + row * width;
     float ss = 0.f, s2 = 0.f;
     if ((width & 3) == 0 && width <= 4 * RA_KEEP * RA_THREADS) {
-        f32x4 keep[RA_KEEP];
+        f32x4 keep[RA_KEEP], xs[RA_KEEP], ws[RA_KEEP];
         const int quads = width >> 2;
 #pragma unroll
         for (int c = 0; c < RA_KEEP; ++c) {
             const int i = threadIdx.x + c * RA_THREADS;
             if (i < quads) {
                 f32x4 v = *(const f32x4*)(yr + 4 * i);
+                if (EARLY) {
+                    xs[c] = *(const f32x4*)(xr + 4 * i);
+                    ws[c] = *(const f32x4*)(w + 4 * i);
+                }
                 if (b) { const f32x4 bb = *(const f32x4*)(b + 4 * i); v[0] += bb[0]; v[1] += bb[1]; v[2] += bb[2]; v[3] += bb[3]; }
                 keep[c] = v;
                 ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
@@ -162,13 +168,17 @@ __global__ __launch_bounds__(RA_THREADS) void rmsnorm_add_kernel(float* __restri
         for (int c = 0; c < RA_KEEP; ++c) {
             const int i = threadIdx.x + c * RA_THREADS;
             if (i < quads) {
-                const f32x4 ww = *(const f32x4*)(w + 4 * i);
-                f32x4 o = *(f32x4*)(xr + 4 * i);
-                o[0] += keep[c][0] * r * ww[0]; o[1] += keep[c][1] * r * ww[1];
-                o[2] += keep[c][2] * r * ww[2]; o[3] += keep[c][3] * r * ww[3];
+                if (!EARLY) {
+                    xs[c] = *(const f32x4*)(xr + 4 * i);
+                    ws[c] = *(const f32x4*)(w + 4 * i);
+                }
+                f32x4 o = xs[c];
+                o[0] += keep[c][0] * r * ws[c][0]; o[1] += keep[c][1] * r * ws[c][1];
+                o[2] += keep[c][2] * r * ws[c][2]; o[3] += keep[c][3] * r * ws[c][3];
                 *(f32x4*)(xr + 4 * i) = o;
                 keep[c] = o;
                 s2 += o[0] * o[0] + o[1] * o[1] + o[2] * o[2] + o[3] * o[3];
+                if (next_w) ws[c] = *(const f32x4*)(next_w + 4 * i);
             }
         }
         if (!next_w) return;
@@ -177,9 +187,8 @@ __global__ __launch_bounds__(RA_THREADS) void rmsnorm_add_kernel(float* __restri
         for (int c = 0; c < RA_KEEP; ++c) {
             const int i = threadIdx.x + c * RA_THREADS;
             if (i < quads) {
-                const f32x4 ww = *(const f32x4*)(next_w + 4 * i);
 #pragma unroll
-                for (int k = 0; k < 4; ++k) nr[4 * i + k] = from_f32<TN>(keep[c][k] * r2 * ww[k]);
+                for (int k = 0; k < 4; ++k) nr[4 * i + k] = from_f32<TN>(keep[c][k] * r2 * ws[c][k]);
             }
         }
         return;
@@ -201,7 +210,10 @@ extern "C" int li_rmsnorm_add(float* x, const float* y, const float* b, const fl
     if (n_rows <= 0) return LI_OK;
     if (width <= 0 || !x || !y || !w || (next_w && !next)) return LI_BAD_ARG;
     if (!next_w) next_dt = DT_F32;
-    DISPATCH_T(next_dt, (rmsnorm_add_kernel<T><<<n_rows, RA_THREADS, 0, stream>>>(x, y, b, w, eps, width, next_w, next_eps, (T*)next)));
+    if (n_rows <= 64)
+        DISPATCH_T(next_dt, (rmsnorm_add_kernel<T, true><<<n_rows, RA_THREADS, 0, stream>>>(x, y, b, w, eps, width, next_w, next_eps, (T*)next)));
+    else
+        DISPATCH_T(next_dt, (rmsnorm_add_kernel<T, false><<<n_rows, RA_THREADS, 0, stream>>>(x, y, b, w, eps, width, next_w, next_eps, (T*)next)));
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
