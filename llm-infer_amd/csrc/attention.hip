@@ -90,14 +90,25 @@ struct WaveAttn {
 
     // Scores of the page's keys (starting at key t0) against this wave's rows, mask, running
     // maximum and sum; leaves the probabilities in s.  This lane's row sees keys lo..hi.
+    // `per` (not 0): every score loses per for every position between the row (at position hi) and its key.
     __device__ __forceinline__ void scores(const v8 (&kf)[2 * KS], f32x16 (&s)[2], int t0, int lo, int hi,
-                                           float scale2, bool masked = true) {
+                                           float scale2, bool masked = true, float per = 0.f) {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[b][r] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) s[b] = mfma32(kf[b * KS + ks], q[ks], s[b]);
+        }
+        if (per != 0.f) {
+            const int lane = threadIdx.x & 63;
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int t = t0 + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    s[b][r] = fmaf(-per, (float)(hi - t), s[b][r]);
+                }
         }
         softmax_step(s, t0, lo, hi, scale2, masked);
     }
@@ -518,7 +529,7 @@ template <class T, int W>
 __global__ __launch_bounds__(64 * W) void attn_decode_kernel(
     const T* __restrict__ q, T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     CachePtrs c, const int* __restrict__ seq_slot, const int* __restrict__ seq_ctx, int H, int K, float scale,
-    int window) {
+    int window, AttnExtras ex) {
     constexpr int OLD = 33;                                   // floats from one output dim to the next in LDS
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -533,7 +544,9 @@ __global__ __launch_bounds__(64 * W) void attn_decode_kernel(
     const int pos = ctx - 1;
     WaveAttn<T> a;
     a.init(live ? q + ((int64_t)b * H + h) * HD : nullptr);
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    if (ex.block > 0) lo = max(lo, pos - pos % ex.block);
+    const float bias_per = (ex.slopes && live) ? ex.slopes[h] / scale : 0.f;    // in the units of the unscaled scores
     const int p_first = lo / PAGE, p_end = pos / PAGE + 1;
     const int per = (p_end - p_first + S - 1) / S;
     const int p0 = p_first + split * per, p1 = min(p_end, p0 + per);
@@ -548,7 +561,7 @@ __global__ __launch_bounds__(64 * W) void attn_decode_kernel(
     if (p0 < p1) a.load_k(kbase + (int64_t)table[p0] * c.page_stride, kf);
     for (int p = p0; p < p1; ++p) {
         a.load_v(vbase + (int64_t)table[p] * c.page_stride, vf);
-        a.scores(kf, s, p * PAGE, lo, live ? pos : -1, scale2, p * PAGE < lo || p * PAGE + PAGE - 1 > pos);
+        a.scores(kf, s, p * PAGE, lo, live ? pos : -1, scale2, p * PAGE < lo || p * PAGE + PAGE - 1 > pos, bias_per);
         if (p + 1 < p1) a.load_k(kbase + (int64_t)table[p + 1] * c.page_stride, kf);
         a.mix(vf, s);
     }
@@ -599,7 +612,14 @@ __global__ __launch_bounds__(64 * W) void attn_decode_kernel(
     }
     if (!live) return;
     if (grid_splits == 1) {
-        const float inv = 1.f / total;
+        float inv;
+        if (ex.sink) {
+            // the sink joins the sum as one more weight, exp(sink - maximum), with nothing to add to the output
+            const float s2 = ex.sink[h] * LOG2E, big = fmaxf(a.m, s2);
+            const float f = (a.m == -INFINITY) ? 0.f : exp2f(a.m - big);
+            inv = f / (total * f + exp2f(s2 - big));
+        } else inv = 1.f / total;
+        if (ex.gate) inv *= 1.f / (1.f + expf(-ex.gate[(int64_t)b * ex.gate_stride + ex.gate_col + h]));
         T* orow = out + ((int64_t)b * H + h) * HD;
 #pragma unroll
         for (int blk = 0; blk < DB; ++blk)
@@ -631,22 +651,27 @@ __global__ __launch_bounds__(64 * W) void attn_decode_kernel(
 // Merge of the splits: M = max m_s, L = sum l_s 2^(m_s - M), o = sum o_s 2^(m_s - M) / L.
 template <class T>
 __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                  T* __restrict__ out, int S) {
+                                  T* __restrict__ out, int S, int H, AttnExtras ex) {
     __shared__ float wgt[64];                        // at most 64 splits
     __shared__ float scratch[16];
     const int64_t row = blockIdx.x;                  // (sequence, head)
+    const int h = (int)(row % H);
     const float* ml = part_ml + row * S * 2;
     const int tid = threadIdx.x;
     const float ms = tid < S ? ml[2 * tid] : -INFINITY;
-    const float M = block_max(ms, scratch);
+    const float s2 = ex.sink ? ex.sink[h] * LOG2E : -INFINITY;         // the sink: one more weight with nothing to add
+    const float M = fmaxf(block_max(ms, scratch), s2);
     const float w = (tid < S && ms != -INFINITY) ? exp2f(ms - M) : 0.f;
-    const float L = block_sum(tid < S ? ml[2 * tid + 1] * w : 0.f, scratch);
+    float L = block_sum(tid < S ? ml[2 * tid + 1] * w : 0.f, scratch);
+    if (ex.sink) L += exp2f(s2 - M);
+    float inv = 1.f / L;
+    if (ex.gate) inv *= 1.f / (1.f + expf(-ex.gate[(row / H) * ex.gate_stride + ex.gate_col + h]));
     if (tid < 64) wgt[tid] = w;
     __syncthreads();
     for (int d = tid; d < HD; d += blockDim.x) {
         float acc = 0.f;
         for (int s = 0; s < S; ++s) acc += part_o[(row * S + s) * HD + d] * wgt[s];
-        out[row * HD + d] = from_f32<T>(acc / L);
+        out[row * HD + d] = from_f32<T>(acc * inv);
     }
 }
 
@@ -753,7 +778,7 @@ extern "C" int li_attn_decode_parts(int splits) { return splits < 1 ? 0 : splits
 template <class T, int W>
 static int launch_decode(const void* q, void* out, float* part_o, float* part_ml, CachePtrs c, const int* seq_slot,
                          const int* seq_ctx, int n_seqs, int H, int K, float scale, int window, int parts,
-                         hipStream_t stream) {
+                         AttnExtras ex, hipStream_t stream) {
     const int G = H / K;
     dim3 grid(n_seqs, K * ((G + 31) / 32), parts), block(64 * W);
     const size_t lds = W > 1 ? (size_t)(W - 1) * (HD * 33 + 64) * sizeof(float) : 0;
@@ -761,10 +786,10 @@ static int launch_decode(const void* q, void* out, float* part_o, float* part_ml
     if (lds > 48 * 1024 &&
         hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return LI_HIP_ERROR;
-    kfn<<<grid, block, lds, stream>>>((const T*)q, (T*)out, part_o, part_ml, c, seq_slot, seq_ctx, H, K, scale, window);
+    kfn<<<grid, block, lds, stream>>>((const T*)q, (T*)out, part_o, part_ml, c, seq_slot, seq_ctx, H, K, scale, window, ex);
     LI_CHECK_LAUNCH();
     if (parts > 1) {
-        attn_merge_kernel<T><<<n_seqs * H, 128, 0, stream>>>(part_o, part_ml, (T*)out, parts);
+        attn_merge_kernel<T><<<n_seqs * H, 128, 0, stream>>>(part_o, part_ml, (T*)out, parts, H, ex);
         LI_CHECK_LAUNCH();
     }
     return LI_OK;
@@ -773,17 +798,20 @@ static int launch_decode(const void* q, void* out, float* part_o, float* part_ml
 extern "C" int li_attn_decode(const void* q, void* out, int dt, const void* k, const void* v, int64_t page_stride,
                               const int* page_table, int max_pages, const int* seq_slot, const int* seq_ctx,
                               int n_seqs, int H, int K, float scale, int window, int splits, float* part_o,
-                              float* part_ml, hipStream_t stream) {
+                              float* part_ml, int key_block, const float* sink, const float* slopes, const float* gate,
+                              int gate_stride, int gate_col, hipStream_t stream) {
     if (check_heads(H, K) || splits < 1 || splits > 64) return LI_BAD_ARG;
+    if (key_block < 0 || !(scale > 0.f) || (gate && (gate_col < 0 || gate_col + H > gate_stride))) return LI_BAD_ARG;
+    const AttnExtras ex{key_block, sink, slopes, gate, gate_stride, gate_col};
     const int w = waves_per_group(splits), parts = splits / w;
     if (parts > 64 || (parts > 1 && (!part_o || !part_ml))) return LI_BAD_ARG;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (n_seqs <= 0) return LI_OK;
     CachePtrs c{k, v, page_stride, page_table, max_pages};
 #define GO(T)                                                                                                      \
-    (w == 4 ? launch_decode<T, 4>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, stream) \
-     : w == 2 ? launch_decode<T, 2>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, stream) \
-              : launch_decode<T, 1>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, stream))
+    (w == 4 ? launch_decode<T, 4>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, ex, stream) \
+     : w == 2 ? launch_decode<T, 2>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, ex, stream) \
+              : launch_decode<T, 1>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, ex, stream))
     return dt == DT_F16 ? GO(f16) : GO(bf16);
 #undef GO
 }

@@ -707,10 +707,15 @@ def attention_prefill(q, kv, meta, n_heads, n_kv_heads, head_dim, scale, window,
 
 
 def attention_decode(q, kv, seq_slot, seq_ctx, n_seqs, n_heads, n_kv_heads, head_dim, scale, window,
-                     splits: int = 1) -> torch.Tensor:
-    """16-bit attention for one new token per sequence; q [B, H, hd]."""
+                     splits: int = 1, block=None, sink=None, slopes=None, gate=None, gate_col: int = 0) -> torch.Tensor:
+    """16-bit attention for one new token per sequence; q [B, H, hd].  ``block``, ``sink``, ``slopes``, ``gate``: as
+    for ``attention_prefill``."""
     k_pages, v_pages, page_stride, page_table = kv
-    _dev(q, k_pages, v_pages, page_table, seq_slot, seq_ctx)
+    _dev(q, k_pages, v_pages, page_table, seq_slot, seq_ctx, sink, slopes, gate)
+    for name, vec in (("sink", sink), ("slopes", slopes)):
+        _need(vec is None or (vec.dtype == torch.float32 and vec.numel() == n_heads and vec.is_contiguous()), f"{name}: float32 [H]")
+    _need(gate is None or (gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] >= n_seqs and gate.stride(1) == 1
+                           and 0 <= gate_col and gate_col + n_heads <= gate.shape[1]), "gate: float32 rows with a column for every head")
     _need(q.dtype in (torch.float16, torch.bfloat16) and q.shape == (n_seqs, n_heads, head_dim), "q: 16-bit [B, H, hd]")
     _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, q.dtype)
     _need(seq_slot.numel() >= n_seqs and seq_ctx.numel() >= n_seqs, "per-sequence arrays too short")
@@ -726,7 +731,8 @@ def attention_decode(q, kv, seq_slot, seq_ctx, n_seqs, n_heads, n_kv_heads, head
     _check(lib.li_attn_decode(
         _ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
         page_table.shape[1], _ptr(seq_slot), _ptr(seq_ctx), n_seqs, n_heads, n_kv_heads, c_float(scale),
-        int(window or 0), splits, _ptr(part_o), _ptr(part_ml), _stream()), "attn_decode")
+        int(window or 0), splits, _ptr(part_o), _ptr(part_ml), int(block or 0), _ptr(sink), _ptr(slopes), _ptr(gate),
+        gate.stride(0) if gate is not None else 0, int(gate_col), _stream()), "attn_decode")
     return out
 
 

@@ -148,6 +148,15 @@ class GatedAttention(Part):
                 shares = min(shares, max(1, span // 128))
         return shares
 
+    def _splits(self, ctx) -> int:
+        """Splits of the keys for the softmax decoder's decode kernel: what the step asks for, but at least two pages a
+        split of what the mask leaves (a power of two)."""
+        splits = ctx.decode_splits(self.n_kv_heads, self.n_heads)
+        for span in (self.block, self.window):
+            if span:
+                splits = min(splits, max(1, span // 128))
+        return 1 << (splits.bit_length() - 1)
+
     def attend(self, h, ctx, views, owns_cache):
         """The heads' gated outputs side by side, [T, H * dv] in the model's type."""
         if owns_cache == self.reads_kv:
@@ -161,11 +170,17 @@ class GatedAttention(Part):
         rows = ops.conv_plain(proj, 0, self.channels, self.conv, views[0].state, ctx) if self.conv_taps else proj
         q = ops.rot_store(rows, self.q_col, self.k_col, self.v_col, getattr(self.position, "inv_freq", None) if self.rot else None,
                           self.rot, ctx.pos, ctx.tok_slot, kv, H, 0 if self.reads_kv else G, d, dv, kv[0].dtype)
-        if self.dtype != torch.float32 and not ctx.is_decode and d == dv and d % 16 == 0 and d <= 256:
-            # prompts of a 16-bit model whose keys and values have one size the kernels take as it is: the softmax
-            # decoder's own prompt kernel (pages through LDS, scores of the next page under the weights of this one)
-            a = ops.attention_prefill(q, kv, ops.prefill_meta(ctx), H, G, d, self.scale, self.window, self.block, self.sinks,
-                                      self.slopes, proj if self.gate else None, self.gate_col)
+        if self.dtype != torch.float32 and d == dv and d % 16 == 0 and d <= 256:
+            # a 16-bit model whose keys and values have one size the kernels take as it is: the softmax decoder's own
+            # kernels (prompts: pages through LDS, scores of the next page under the weights of this one; decode steps:
+            # a wave per (sequence, key/value head, split of the keys that the mask leaves))
+            gate = proj if self.gate else None
+            if ctx.is_decode:
+                a = ops.attention_decode(q, kv, ctx.seq_slot, ctx.seq_ctx, ctx.n_seqs, H, G, d, self.scale, self.window,
+                                         self._splits(ctx), self.block, self.sinks, self.slopes, gate, self.gate_col)
+            else:
+                a = ops.attention_prefill(q, kv, ops.prefill_meta(ctx), H, G, d, self.scale, self.window, self.block, self.sinks,
+                                          self.slopes, gate, self.gate_col)
             return a.view(a.shape[0], H * dv)
         sixteen = self.dtype != torch.float32 and ops.diff_attention_fits(d, dv)
         return ops.diff_attention(q, kv, ctx.pos, ctx.tok_slot, H, G, 1, d, dv, self.scale, self.block, self.window, 0.0, None, 1.0,
