@@ -65,15 +65,15 @@ TINY_B = config(72, 97, [
     layer(convolved(1, 1, 8, 40, 7, taps=5), dense(40, limit=3.0)),
     layer(rotary(4, 4, 16, 1000, dims=0), moe(4, 4, 8)),
     layer(convolved(1, 1, 8, 40, 33, taps=1, kv_from=0), moe(9, 3, 16, shared=16)),
-    layer(rotary(6, 2, 48, 33, dims=16, base=77.0, scaling=(8.0, 1.0, 4.0, 32)), dense(24)),
-    layer(rotary(6, 2, 48, 90, dims=16, base=77.0, scaling=(8.0, 1.0, 4.0, 32), kv_from=3), None),
+    layer(rotary(6, 2, 48, 33, dims=16, base=77.0, scaling=(6.0, 1.0, 3.0, 32)), dense(24)),
+    layer(rotary(6, 2, 48, 90, dims=16, base=77.0, scaling=(6.0, 1.0, 3.0, 32), kv_from=3), None),
 ], eps=1e-4, scale=1.0, logit_scale=3.0)
 
 # sizes of real layers, few of them: eight heads of 64 on two key heads, sixteen heads of 128 on one; windows and chunks
 # beyond a page
 TINY_C = config(256, 211, [
     layer(convolved(16, 1, 128, 64, 130, taps=4), moe(4, 2, 96, shared=64)),
-    layer(rotary(8, 2, 64, 100, base=1e6, scaling=(8.0, 1.0, 4.0, 128)), dense(320)),
+    layer(rotary(8, 2, 64, 100, base=2e5, scaling=(16.0, 1.0, 2.0, 128)), dense(320)),
     layer(convolved(16, 1, 128, 64, 130, taps=4, kv_from=0), dense(128, limit=7.0)),
 ], eps=1e-5, scale=3.0, logit_scale=0.5)
 

@@ -246,7 +246,7 @@ SCHEDULES = {
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("mixer", [
     M.rotary(3, 1, 20, 9, dims=12, base=500.0),                                  # a padded head, a window below a page
-    M.rotary(8, 2, 64, 100, scaling=(8.0, 1.0, 4.0, 128), base=1e6),             # a window across pages, stretched frequencies
+    M.rotary(8, 2, 64, 100, scaling=(16.0, 1.0, 2.0, 128), base=2e5),             # a window across pages, stretched frequencies
     M.rotary(4, 4, 16, 1000, dims=0),                                            # no rotation, a window never reached
     M.rotary(2, 1, 48, 64, dims=48, scaling=(2.0, 1.0, 2.0, 40)),                # window = page
     M.convolved(4, 2, 16, 24, 50, taps=2),                                       # values wider than keys
