@@ -53,6 +53,10 @@ extern "C" int li_scale_values(float* x, int64_t n, float s, hipStream_t stream)
 // the values are not.  q goes to q_out [T, H, DP] in the cache's type (DP = d rounded up to 16, zeros behind d),
 // k (padded likewise) and v into the page of position p in matrix-operand order (common.h; one map of keys).
 // G_store 0: only q (a layer that reads another layer's keys and values).
+// `conv_w` not null (float32 [channels, taps]): what is read of the rows is first convolved over time, channel by
+// channel (column c of the rows is channel c; the last tap is the token's own), y_t = sum_j w[c][j] u_(t - taps + 1 + j):
+// inputs before the first token that a sequence brings to this step come from `hist` [slots, taps - 1, channels] (the
+// last inputs of the steps before, oldest first; before position 0 they are zero), which this kernel only reads.
 // ---------------------------------------------------------------------------
 struct StorePages {
     void* k;
@@ -68,17 +72,34 @@ template <class T>
 __global__ void rot_store_kernel(const float* __restrict__ rows, int stride, int q_col, int k_col, int v_col,
                                  const float* __restrict__ inv_freq, int rot, const int* __restrict__ pos,
                                  const int* __restrict__ tok_slot, T* __restrict__ q_out, StorePages pg, int H, int G,
-                                 int d, int dv) {
+                                 int d, int dv, const float* __restrict__ conv_w, int taps, const float* __restrict__ hist,
+                                 int channels) {
     __shared__ float cs[2 * ROT_MAX_PAIRS];               // cos and sin of the token's angles, one pair of them a pair of dimensions
     const int t = blockIdx.x, p = pos[t], DP = round_up(d, 16), half = rot >> 1;
     for (int j = threadIdx.x; j < half; j += blockDim.x) sincosf((float)p * inv_freq[j], &cs[2 * j + 1], &cs[2 * j]);
     if (half) __syncthreads();
     const float* row = rows + (int64_t)t * stride;
+    const int slot = tok_slot[t];
+    // how many tokens before this one its sequence has in this step (at most taps - 1 matter)
+    int inside = 0;
+    if (conv_w) while (inside < taps - 1 && t - inside - 1 >= 0 && tok_slot[t - inside - 1] == slot) ++inside;
+    const float* h = conv_w ? hist + (int64_t)slot * (taps - 1) * channels : nullptr;
+    auto value = [&](int c) {                             // column c of this token's row, convolved where asked
+        if (!conv_w) return row[c];
+        float acc = 0.f;
+        for (int back = 0; back < taps; ++back) {
+            float u = 0.f;
+            if (back <= inside) u = row[c - (int64_t)back * stride];
+            else if (p - back >= 0) u = h[(int64_t)(taps - 1 - (back - inside)) * channels + c];
+            acc += conv_w[(int64_t)c * taps + (taps - 1 - back)] * u;
+        }
+        return acc;
+    };
     T* kp = nullptr;
     T* vp = nullptr;
     const int off = p % PAGE;
     if (G > 0) {
-        const int page = pg.page_table[(int64_t)tok_slot[t] * pg.max_pages + p / PAGE];
+        const int page = pg.page_table[(int64_t)slot * pg.max_pages + p / PAGE];
         kp = (T*)pg.k + (int64_t)page * pg.page_stride;
         vp = (T*)pg.v + (int64_t)page * pg.page_stride;
     }
@@ -87,21 +108,21 @@ __global__ void rot_store_kernel(const float* __restrict__ rows, int stride, int
         if (e < n_qk) {
             const int u = e / DP, i = e - u * DP;
             const bool is_q = u < H;
-            const float* src = row + (is_q ? q_col + u * d : k_col + (u - H) * d);
+            const int src = is_q ? q_col + u * d : k_col + (u - H) * d;
             float val = 0.f;
             if (i < d) {
-                val = src[i];
+                val = value(src + i);
                 if (i < rot) {
                     const int j = i < half ? i : i - half;
                     const float c_ = cs[2 * j], s_ = cs[2 * j + 1];
-                    val = i < half ? val * c_ - src[i + half] * s_ : val * c_ + src[i - half] * s_;
+                    val = i < half ? val * c_ - value(src + i + half) * s_ : val * c_ + value(src + i - half) * s_;
                 }
             }
             if (is_q) q_out[((int64_t)t * H + u) * DP + i] = from_f32<T>(val);
             else kp[(int64_t)(u - H) * k_head_elems(DP) + k_offset(off, i, DP)] = from_f32<T>(val);
         } else {
             const int r = e - n_qk, g = r / dv, j = r - g * dv;
-            vp[(int64_t)g * v_head_elems(dv) + v_offset(off, j, dv)] = from_f32<T>(row[v_col + r]);
+            vp[(int64_t)g * v_head_elems(dv) + v_offset(off, j, dv)] = from_f32<T>(value(v_col + r));
         }
     }
 }
@@ -109,17 +130,24 @@ __global__ void rot_store_kernel(const float* __restrict__ rows, int stride, int
 extern "C" int li_rot_store(const float* rows, int stride, int q_col, int k_col, int v_col, const float* inv_freq, int rot,
                             const int* pos, const int* tok_slot, void* q_out, void* k_pages, void* v_pages,
                             int64_t page_stride, const int* page_table, int max_pages, int dt, int n, int H, int G_store,
-                            int d, int dv, hipStream_t stream) {
+                            int d, int dv, const float* conv_w, int taps, const float* hist, int channels,
+                            hipStream_t stream) {
     if (n <= 0) return LI_OK;
     if (H <= 0 || G_store < 0 || d <= 0 || dv <= 0 || rot < 0 || rot > d || (rot & 1) || (rot && !inv_freq)) return LI_BAD_ARG;
     if (rot > 2 * ROT_MAX_PAIRS) return LI_UNSUPPORTED;
     if (q_col < 0 || q_col + H * d > stride) return LI_BAD_ARG;
     if (G_store && (k_col < 0 || v_col < 0 || k_col + G_store * d > stride || v_col + G_store * dv > stride)) return LI_BAD_ARG;
+    if (conv_w) {
+        // every column that is read is a channel of the convolution
+        const int last = G_store ? (k_col + G_store * d > v_col + G_store * dv ? k_col + G_store * d : v_col + G_store * dv) : 0;
+        if (taps < 1 || taps > 16 || (taps > 1 && !hist) || channels > stride || q_col + H * d > channels || last > channels)
+            return LI_BAD_ARG;
+    }
     StorePages pg{k_pages, v_pages, page_stride, page_table, max_pages};
     const int total = (H + G_store) * round_up(d, 16) + G_store * dv;
     dim3 grid(n, n >= 512 ? 1 : (total + 255) / 256);
     DISPATCH_T(dt, (rot_store_kernel<T><<<grid, 256, 0, stream>>>(rows, stride, q_col, k_col, v_col, inv_freq, rot, pos, tok_slot,
-                                                              (T*)q_out, pg, H, G_store, d, dv)));
+                                                              (T*)q_out, pg, H, G_store, d, dv, conv_w, taps, hist, channels)));
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

@@ -400,20 +400,14 @@ extern "C" int li_conv_add(const float* in, int stride, int col0, const float* w
     return LI_OK;
 }
 
-// The same convolution alone: no activation, the input not added, float32 out (what a mixer convolves behind its own
-// input product before anything else is done to it).
-extern "C" int li_conv_plain(const float* in, int stride, int col0, const float* w, const float* b, float* hist,
-                             const int* pos, const int* tok_slot, const int* seq_slot, const int* seq_qstart,
-                             const int* seq_qlen, float* out, int n_tokens, int n_seqs, int channels, int taps,
-                             hipStream_t stream) {
-    if (n_tokens <= 0) return LI_OK;
-    if (channels <= 0 || taps < 1 || taps > CONV_MAX_TAPS) return LI_BAD_ARG;
-    dim3 cgrid(n_tokens, (channels + 255) / 256);
-    conv_silu_kernel<float, false, false><<<cgrid, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, out, channels, taps);
-    if (taps > 1) {
-        dim3 grid(n_seqs, (channels + 255) / 256);
-        conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);
-    }
+// A sequence's last taps - 1 inputs brought up to date alone (for a kernel that convolves while it does something else
+// and only reads the history).
+extern "C" int li_conv_history(const float* in, int stride, int col0, float* hist, const int* seq_slot, const int* seq_qstart,
+                               const int* seq_qlen, int n_seqs, int channels, int taps, hipStream_t stream) {
+    if (n_seqs <= 0 || taps <= 1) return LI_OK;
+    if (channels <= 0 || taps > CONV_MAX_TAPS) return LI_BAD_ARG;
+    dim3 grid(n_seqs, (channels + 255) / 256);
+    conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

@@ -1782,34 +1782,31 @@ def scale_values(x: torch.Tensor, s: float) -> torch.Tensor:
     return x
 
 
-def conv_plain(rows, col0, channels, weight, history, ctx) -> torch.Tensor:
-    """A causal convolution per channel over ``channels`` columns of the float32 ``rows`` from ``col0`` on, alone: weight
-    float32 [channels, taps] (last column: the current token), no bias, no activation; ``history`` float32
-    [slots, taps - 1, channels] holds every sequence's last inputs and is brought up to date.  Returns float32
-    [T, channels]."""
-    _dev(rows, weight, history)
+def conv_history(rows, col0, channels, taps, history, ctx) -> None:
+    """Brings ``history`` (float32 [slots, taps - 1, channels]: every sequence's last inputs of a causal convolution) up
+    to date with the step's ``rows`` (float32, the channels from column ``col0`` on); for a kernel that convolves on the
+    way to something else and only reads the history."""
+    _dev(rows, history)
     _f32_rows(rows, "conv rows")
-    t, taps = rows.shape[0], weight.shape[1]
-    _need(weight.dtype == torch.float32 and weight.shape == (channels, taps) and 1 <= taps <= 16, "conv weight: float32 [channels, taps <= 16]")
-    _need(0 <= col0 and col0 + channels <= rows.shape[1], "conv: columns beyond the rows")
+    _need(1 <= taps <= 16 and 0 <= col0 and col0 + channels <= rows.shape[1], "conv history: columns within the rows, up to 16 taps")
     _need(history.dtype == torch.float32 and history.dim() == 3 and tuple(history.shape[1:]) == (max(taps - 1, 1), channels),
           "conv history: float32 [slots, taps - 1, channels]")
-    _i32(ctx.pos, t, "positions")
-    _i32(ctx.tok_slot, t, "slots")
-    seq_slot, qstart, qlen = _seq_arrays(ctx, t)
-    out = torch.empty((t, channels), dtype=torch.float32, device=rows.device)
-    _check(hybrid().li_conv_plain(_ptr(rows), rows.shape[1], col0, _ptr(weight), None, _ptr(history), _ptr(ctx.pos),
-                                  _ptr(ctx.tok_slot), _ptr(seq_slot), _ptr(qstart), _ptr(qlen), _ptr(out), t, ctx.n_seqs, channels,
-                                  taps, _stream()), "conv_plain")
-    return out
+    seq_slot, qstart, qlen = _seq_arrays(ctx, rows.shape[0])
+    _check(hybrid().li_conv_history(_ptr(rows), rows.shape[1], col0, _ptr(history), _ptr(seq_slot), _ptr(qstart), _ptr(qlen),
+                                    ctx.n_seqs, channels, taps, _stream()), "conv_history")
 
 
-def rot_store(rows, q_col, k_col, v_col, inv_freq, rot, pos, tok_slot, kv, n_heads, n_kv_store, d, dv, q_dtype=None) -> torch.Tensor:
+def rot_store(rows, q_col, k_col, v_col, inv_freq, rot, pos, tok_slot, kv, n_heads, n_kv_store, d, dv, q_dtype=None,
+              conv=None) -> torch.Tensor:
     """From float32 rows with a token's q heads [H, d] from column ``q_col``, k heads [G, d] from ``k_col`` and values
     [G, dv] from ``v_col`` (it may equal ``k_col``: the values are the keys before their rotation): q and k turned by
     position in their first ``rot`` dimensions, dimension i paired with i + rot / 2, angle pos * inv_freq[i]; k and v
     into the pages in matrix-operand order (one map of keys, padded to a multiple of 16).  ``n_kv_store`` 0: nothing
-    is stored (``kv`` may be None, ``q_dtype`` says q's type).  Returns q [T, H, DP] in the cache's type."""
+    is stored (``kv`` may be None, ``q_dtype`` says q's type).  ``conv`` (weight float32 [channels, taps], history float32
+    [slots, taps - 1, channels]): column c of the rows is channel c of a causal convolution over time that everything
+    read passes first (the last tap is the token's own; inputs before the step's first token of a sequence come from
+    the history, which is only read: ``conv_history`` brings it up to date afterwards).  Returns q [T, H, DP] in the
+    cache's type."""
     _dev(rows, inv_freq, pos, tok_slot)
     _f32_rows(rows, "rot_store rows")
     t = rows.shape[0]
@@ -1829,10 +1826,21 @@ def rot_store(rows, q_col, k_col, v_col, inv_freq, rot, pos, tok_slot, kv, n_hea
         k_pages = v_pages = page_table = None
         page_stride = max_pages = 0
         _need(q_dtype in DT, "rot_store: q's type")
+    conv_w = hist = None
+    taps = channels = 0
+    if conv is not None:
+        conv_w, hist = conv
+        _dev(conv_w, hist)
+        channels, taps = conv_w.shape
+        _need(conv_w.dtype == torch.float32 and conv_w.is_contiguous() and 1 <= taps <= 16 and channels <= rows.shape[1],
+              "rot_store: conv weight float32 [channels, taps <= 16] for the first columns of the rows")
+        _need(hist.dtype == torch.float32 and hist.dim() == 3 and tuple(hist.shape[1:]) == (max(taps - 1, 1), channels),
+              "rot_store: conv history float32 [slots, taps - 1, channels]")
     q = torch.empty((t, n_heads, dp), dtype=q_dtype, device=rows.device)
     _check(hybrid().li_rot_store(_ptr(rows), rows.shape[1], q_col, k_col, v_col, _ptr(inv_freq), rot, _ptr(pos), _ptr(tok_slot),
                                  _ptr(q), _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table), max_pages,
-                                 DT[q_dtype], t, n_heads, n_kv_store, d, dv, _stream()), "rot_store")
+                                 DT[q_dtype], t, n_heads, n_kv_store, d, dv, _ptr(conv_w), taps, _ptr(hist), channels,
+                                 _stream()), "rot_store")
     return q
 
 

@@ -167,9 +167,12 @@ class GatedAttention(Part):
             proj = ops.linear(h, self.w_in, ops.EPI_BIAS, out_dtype=torch.float32, params=self.b_in)
         else:
             proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
-        rows = ops.conv_plain(proj, 0, self.channels, self.conv, views[0].state, ctx) if self.conv_taps else proj
-        q = ops.rot_store(rows, self.q_col, self.k_col, self.v_col, getattr(self.position, "inv_freq", None) if self.rot else None,
-                          self.rot, ctx.pos, ctx.tok_slot, kv, H, 0 if self.reads_kv else G, d, dv, kv[0].dtype)
+        # the convolution rides in the kernel that turns and stores; the history is brought up to date behind it
+        conv = (self.conv, views[0].state) if self.conv_taps else None
+        q = ops.rot_store(proj, self.q_col, self.k_col, self.v_col, getattr(self.position, "inv_freq", None) if self.rot else None,
+                          self.rot, ctx.pos, ctx.tok_slot, kv, H, 0 if self.reads_kv else G, d, dv, kv[0].dtype, conv)
+        if self.conv_taps > 1:
+            ops.conv_history(proj, 0, self.channels, self.conv_taps, views[0].state, ctx)
         if self.dtype != torch.float32 and d == dv and d % 16 == 0 and d <= 256:
             # a 16-bit model whose keys and values have one size the kernels take as it is: the softmax decoder's own
             # kernels (prompts: pages through LDS, scores of the next page under the weights of this one; decode steps:

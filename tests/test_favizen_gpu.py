@@ -161,11 +161,13 @@ def test_experts_by_table(lib):
 
 
 @pytest.mark.parametrize("taps", [1, 2, 5])
-def test_convolution_behind_a_product_in_portions(lib, taps):
-    """Portions shorter than the convolution's reach, two sequences at once, a slot used again."""
+def test_convolution_on_the_way_into_the_cache_in_portions(lib, taps):
+    """The store kernel's convolution: portions shorter than its reach, two sequences at once, a slot used again; q as it
+    comes back is compared (keys and values take the same path and are checked through the mixers)."""
     from llm_infer_amd.kernels import ops
     g = torch.Generator().manual_seed(4)
-    C, extra = 10, 3
+    H, d, extra = 2, 5, 3
+    C = H * d
     w = torch.randn(C, taps, generator=g)
     u = {r: torch.randn(n, C + extra, generator=g) for r, n in (("a", 11), ("b", 6), ("c", 4))}
     hist = torch.full((4, max(taps - 1, 1), C), 7.0, device=DEV)           # what an earlier sequence left
@@ -178,12 +180,15 @@ def test_convolution_behind_a_product_in_portions(lib, taps):
                 hist[slot[r]] = 0.0                                        # the cache clears a slot's state when it hands it out
         ctx = step_context([slot[r] for r in rs], [at[r] for r in rs], [[0] * step[r] for r in rs])
         x = torch.cat([u[r][at[r]:at[r] + step[r]] for r in rs]).to(DEV)
-        out = ops.conv_plain(x, extra, C, w.to(DEV), hist, ctx).cpu()
+        q = ops.rot_store(x, 0, 0, 0, None, 0, ctx.pos, ctx.tok_slot, None, H, 0, d, d, torch.float32, (w.to(DEV), hist))
+        ops.conv_history(x, 0, C, taps, hist, ctx)
+        out = q[:, :, :d].reshape(-1, C).cpu()
+        assert float(q[:, :, d:].abs().max()) == 0.0                        # zeros behind a head's own dimensions
         for r, part in zip(rs, out.split([step[r] for r in rs])):
             got[r].append(part)
             at[r] += step[r]
     for r in u:
-        ref = P.causal_conv(u[r][:, extra:].double(), w.double())
+        ref = P.causal_conv(u[r][:, :C].double(), w.double())
         assert error(torch.cat(got[r]), ref) < 1e-6, r
 
 
